@@ -5,7 +5,7 @@ Plain ``hipcc`` invocations (no hipify, no torch JIT cache): every ``csrc/*.hip`
 source, the headers or the flags changes), then one link step produces the shared library next to this file, so it
 travels with the repository snapshot to the GPU box.
 
-    python -m llmctl.ops.build [-j N] [--force] [--arch gfx950] [--save-temps]
+    python -m llmctl.ops.build [-j N] [--force] [--arch gfx950]
 """
 
 from __future__ import annotations
@@ -36,14 +36,12 @@ def hipcc() -> str:
     return str(p) if p.exists() else "hipcc"
 
 
-def compile_flags(arch: str, save_temps: bool = False):
+def compile_flags(arch: str):
     incs, _ = torch_paths()
     flags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={arch}", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
              "-D_GLIBCXX_USE_CXX11_ABI=1", "-Wno-unused-result", "-Wno-deprecated-declarations",
              "-Wno-return-type", f"-I{CSRC}"]
     flags += [f"-I{i}" for i in incs]
-    if save_temps:
-        flags += ["-save-temps=obj"]
     # diagnostic builds only (e.g. LLMCTL_BUILD_DEFINES="LLMCTL_STAMP LLMCTL_STAMP_EXP=2" for the
     # persistent GEMM's cycle stamps, tools/gemm_stamps.py); the production library sets none
     flags += [f"-D{d}" for d in os.environ.get("LLMCTL_BUILD_DEFINES", "").split() if d]
@@ -79,10 +77,10 @@ def _needs(src: Path, obj: Path, flags) -> bool:
     return not (obj.exists() and key.exists() and key.read_text() == _digest(src, flags))
 
 
-def build(arch: str = "gfx950", jobs: int = 0, force: bool = False, save_temps: bool = False, verbose: bool = True) -> Path:
+def build(arch: str = "gfx950", jobs: int = 0, force: bool = False, verbose: bool = True) -> Path:
     BUILD.mkdir(parents=True, exist_ok=True)
     srcs = sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
-    flags = compile_flags(arch, save_temps)
+    flags = compile_flags(arch)
     todo = []
     objs = []
     for s in srcs:
@@ -127,9 +125,8 @@ def main(argv=None):
     ap.add_argument("--arch", default=os.environ.get("PYTORCH_ROCM_ARCH", "gfx950").split(";")[0])
     ap.add_argument("-j", "--jobs", type=int, default=0)
     ap.add_argument("--force", action="store_true")
-    ap.add_argument("--save-temps", action="store_true")
     a = ap.parse_args(argv)
-    build(a.arch, a.jobs, a.force, a.save_temps)
+    build(a.arch, a.jobs, a.force)
 
 
 if __name__ == "__main__":

@@ -1329,8 +1329,7 @@ __global__ __launch_bounds__(NT4, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
 // buffer descriptors are dead.  The earlier, unpeeled form held both descriptor sets through the
 // loop (SGPRs spilled to VGPR lanes) and gave intermittent wrong rows; the peeled form fixed that
 // empirically (every test since), but the root cause is NOT pinned down: the suspected VALU write
-// of an SGPR (v_readlane reload) ahead of an inline-asm buffer_load was not confirmed --
-// tools/sgpr_hazard_check.py found only SALU writers ahead of those loads.  K >= 256.
+// of an SGPR (v_readlane reload) ahead of an inline-asm buffer_load was not confirmed.  K >= 256.
 // Phase schedule: the one-shot 4-wave kernel's.
 // STAMP (diagnostic build only: compile with -DLLMCTL_STAMP, then knob gemm_stamp_ptr=<device u32
 // buffer>): lane 0 of every wave records s_memtime (low 32 bits) at the start of every phase of its
