@@ -33,12 +33,20 @@ def resolve_checkpoint_dir(path: str) -> Optional[Path]:
 
 def load_model(path: str, device=None, dtype=torch.bfloat16, pc: Optional[ParallelContext] = None,
                seed: int = 0) -> Tuple[DecoderLM, ModelConfig, Optional[Path]]:
+    from llmctl.models.registry import family_of_config
+
     ck = resolve_checkpoint_dir(path)
+    cfg = get_model_config(path) if ck is None else ModelConfig.from_file(ck / "config.json")
+    fam = family_of_config(cfg)
+    if fam is not None:  # a registered family builds / loads itself (no TP / PP sharding)
+        if pc is not None and (pc.tp_size > 1 or pc.layer_start or pc.layer_end is not None):
+            raise NotImplementedError(f"{cfg.architecture}: tensor / pipeline parallel serving")
+        if ck is None:
+            return fam.build(cfg, device=device, dtype=dtype, seed=seed), cfg, None
+        return fam.load(ck, cfg, device=device, dtype=dtype), cfg, ck
     if ck is None:
-        cfg = get_model_config(path)
         model = build_model(cfg, device=device, dtype=dtype, pc=pc, seed=seed)
         return model, cfg, None
-    cfg = ModelConfig.from_file(ck / "config.json")
     from llmctl.io.checkpoint import _global_name, load_full_state_dict, shard_tp
 
     full = load_full_state_dict(ck, cfg)

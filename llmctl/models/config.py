@@ -143,10 +143,15 @@ class ModelConfig:
         return cls(**kw)
 
     @classmethod
-    def from_file(cls, path: str | Path) -> "ModelConfig":
+    def from_file(cls, path: str | Path):
         path = Path(path)
         if path.suffix == ".json":
             data = json.loads(path.read_text())
+            from .registry import family_of
+
+            fam = family_of(data)  # another model family: its own config class
+            if fam is not None:
+                return fam.config_cls.from_dict(data)
         else:
             from llmctl.config.toml_io import load_toml
 
@@ -270,6 +275,11 @@ def get_model_config(name_or_path: str) -> ModelConfig:
     if p.suffix in (".json", ".toml") and p.exists():
         return ModelConfig.from_file(p)
     key = name_or_path.lower()
+    if key.startswith("lenitar-"):  # lenitar-w<width>-l<layers>[-h<heads>]: random-init template
+        from .lenitar import lenitar_template
+
+        kv = {p[0]: int(p[1:]) for p in key.split("-")[1:] if p[1:].isdigit()}
+        return lenitar_template(width=kv.get("w", 256), layers=kv.get("l", 4), heads=kv.get("h", 4))
     if key in ALIASES:
         t, s = ALIASES[key]
         return ModelConfig.from_dict(MODEL_TEMPLATES[t][s])

@@ -138,15 +138,7 @@ class MoEMLP(nn.Module):
                     o += n
             ye = torch.cat(outs, 0).index_select(0, dst) if outs else xe.new_zeros((0, h))
         else:
-            outs = []
-            o = 0
-            for e, n in enumerate(local_counts):
-                if n == 0:
-                    continue
-                seg = xe[o:o + n]
-                o += n
-                outs.append(linear(ops.swiglu(linear(seg, self.experts_up[e])), self.experts_down[e]))
-            ye = torch.cat(outs, 0) if outs else xe.new_zeros((0, h))
+            ye = run_expert_segments(xe, local_counts, self.experts_up, self.experts_down)
         if self.ep > 1:
             inv = torch.empty_like(perm_t)
             inv[perm_t] = torch.arange(perm_t.numel(), device=x.device)
@@ -174,6 +166,59 @@ class MoEMLP(nn.Module):
         dst = torch.cat(idx).to(xe.device, non_blocking=True) if idx else torch.zeros(0, dtype=torch.long,
                                                                                        device=xe.device)
         return dst, padded
+
+
+def run_expert_segments(xe: torch.Tensor, counts: List[int], ups, downs, act=None) -> torch.Tensor:
+    """``down_e(act(up_e(x)))`` on each expert's contiguous row segment of ``xe`` (rows sorted by
+    expert, ``counts[e]`` rows each)."""
+    act = act or ops.swiglu
+    outs, o = [], 0
+    for e, n in enumerate(counts):
+        if n == 0:
+            continue
+        seg = xe[o:o + n]
+        o += n
+        outs.append(linear(act(linear(seg, ups[e])), downs[e]))
+    return torch.cat(outs, 0) if outs else xe.new_zeros((0, downs[0].shape[0]))
+
+
+class GroupLimitedMoE(nn.Module):
+    """Routed SwiGLU experts with sigmoid scores and group-limited choice (serving forward).
+
+    Router logits are an fp32 product; scores ``sigmoid(z)``; experts form ``groups`` equal groups of
+    neighbours, a group is scored by the sum of its two best experts, only the ``keep`` best groups are
+    eligible and the ``top`` best eligible experts are used, weighted by their own scores (no
+    renormalisation).  Token copies are sorted by expert and run through per-expert GEMMs on
+    contiguous segments (the dispatch of :class:`MoEMLP`); the weighted sum is accumulated in fp32."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, groups: int, keep: int, device=None, dtype=None):
+        super().__init__()
+        if experts % groups or not (0 < keep <= groups) or not (0 < top <= keep * (experts // groups)):
+            raise ValueError("router: experts must split into equal groups and top must fit the kept groups")
+        self.E, self.top, self.groups, self.keep, self.ff = experts, top, groups, keep, ff
+        kw = dict(device=device, dtype=dtype)
+        self.w_router = nn.Parameter(torch.empty(experts, width, device=device, dtype=torch.float32))
+        self.experts_up = nn.ParameterList([nn.Parameter(torch.empty(2 * ff, width, **kw)) for _ in range(experts)])
+        self.experts_down = nn.ParameterList([nn.Parameter(torch.empty(width, ff, **kw)) for _ in range(experts)])
+        with torch.no_grad():
+            self.w_router.normal_(0.0, 0.02)
+            for p in list(self.experts_up) + list(self.experts_down):
+                p.normal_(0.0, 0.02)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [T, width] -> fp32 [T, width]."""
+        from llmctl.ops import hybrid as hops
+
+        T = x.shape[0]
+        topi, topw = hops.group_topk_router(torch.nn.functional.linear(x.float(), self.w_router), self.top,
+                                            self.groups, self.keep)
+        flat = topi.reshape(-1)
+        counts = torch.bincount(flat, minlength=self.E).tolist()  # the layer's one host sync
+        order = torch.argsort(flat, stable=True)
+        tok = torch.div(order, self.top, rounding_mode="floor")
+        ye = run_expert_segments(x.index_select(0, tok), counts, self.experts_up, self.experts_down, hops.swiglu_any)
+        w = topw.reshape(-1).index_select(0, order).unsqueeze(-1)
+        return torch.zeros(T, x.shape[1], dtype=torch.float32, device=x.device).index_add_(0, tok, ye.float() * w)
 
 
 def expert_param_global_name(name: str, module_e0: int) -> str:

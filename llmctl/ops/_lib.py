@@ -59,6 +59,23 @@ def native():
     return torch.ops.llmctl
 
 
+HYBRID_LIB_PATH = Path(__file__).resolve().parent / "_llmctl_hybrid.so"
+_hybrid_loaded = False
+
+
+def native_hybrid():
+    """The ``torch.ops.llmctl_hybrid`` namespace (kernels of the hybrid sequence mixers, their own
+    library so that a model of that family needs only it built); raises if it is absent."""
+    global _hybrid_loaded
+    if not _hybrid_loaded:
+        if not HYBRID_LIB_PATH.exists():
+            raise RuntimeError(f"llmctl hybrid-mixer kernels are required for GPU tensors but {HYBRID_LIB_PATH} "
+                               "is not built (run `python -m llmctl.ops.build --group hybrid`)")
+        torch.ops.load_library(str(HYBRID_LIB_PATH))
+        _hybrid_loaded = True
+    return torch.ops.llmctl_hybrid
+
+
 def use_native(t: torch.Tensor) -> bool:
     if not t.is_cuda:
         return False

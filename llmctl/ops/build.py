@@ -40,7 +40,9 @@ def compile_flags(arch: str):
     incs, _ = torch_paths()
     flags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={arch}", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
              "-D_GLIBCXX_USE_CXX11_ABI=1", "-Wno-unused-result", "-Wno-deprecated-declarations",
-             "-Wno-return-type", f"-I{CSRC}"]
+             "-Wno-return-type", f"-I{CSRC}",
+             # no packed-fp32 VALU forms (some of them have given wrong results on this part)
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     flags += [f"-I{i}" for i in incs]
     # diagnostic builds only (e.g. LLMCTL_BUILD_DEFINES="LLMCTL_STAMP LLMCTL_STAMP_EXP=2" for the
     # persistent GEMM's cycle stamps, tools/gemm_stamps.py); the production library sets none

@@ -168,3 +168,74 @@ class PagedKVCache:
     @property
     def nbytes(self) -> int:
         return self.k.numel() * self.k.element_size() * 2
+
+
+class StateSlotManager:
+    """Slots of the recurrent-state pools: one per live sequence, taken at admission and given back
+    when the sequence finishes or is preempted.  A slot's content is never cleared: a sequence that
+    starts at position 0 ignores what the slot holds."""
+
+    def __init__(self, num_slots: int):
+        self._num = num_slots
+        self.free_list = list(range(num_slots - 1, -1, -1))
+        self.owner: Dict[int, int] = {}
+
+    def alloc(self, seq: int) -> bool:
+        if seq in self.owner:
+            raise RuntimeError("sequence already holds a state slot")
+        if not self.free_list:
+            return False
+        self.owner[seq] = self.free_list.pop()
+        return True
+
+    def free(self, seq: int) -> None:
+        s = self.owner.pop(seq, None)
+        if s is not None:
+            self.free_list.append(s)
+
+    def slot(self, seq: int) -> int:
+        return self.owner[seq]
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free_list)
+
+    @property
+    def num_slots(self) -> int:
+        return self._num
+
+
+class HybridCache:
+    """The cache of a model whose layers mix differently: per layer either a paged pool of cache rows
+    (``("latent", row_width)``: ``[num_blocks, block_size, row_width]``, addressed through the same
+    block tables as a K/V cache) or fp32 recurrent-state pools (``("state", [shape, ...])``:
+    ``[num_slots, *shape]`` each, addressed by the sequence's slot).  Layers may differ in size."""
+
+    def __init__(self, kinds, num_blocks: int, block_size: int, num_slots: int, dtype=torch.bfloat16, device=None):
+        self.num_blocks, self.block_size, self.num_slots = num_blocks, block_size, num_slots
+        self._layers = []
+        for kind, spec in kinds:
+            if kind == "latent":
+                self._layers.append(torch.zeros(num_blocks, block_size, int(spec), dtype=dtype, device=device))
+            elif kind == "state":
+                self._layers.append(tuple(torch.zeros((num_slots,) + tuple(s), dtype=torch.float32, device=device)
+                                          for s in spec))
+            else:
+                raise ValueError(f"unknown cache kind {kind!r}")
+        self.has_state = any(k == "state" for k, _ in kinds)
+        self.slots = StateSlotManager(num_slots) if self.has_state else None
+
+    def layer(self, i: int):
+        return self._layers[i]
+
+    @staticmethod
+    def bytes_per_block(kinds, block_size: int, dtype_bytes: int) -> int:
+        return max(sum(int(s) for k, s in kinds if k == "latent") * block_size * dtype_bytes, 1)
+
+    @property
+    def nbytes(self) -> int:
+        n = 0
+        for l in self._layers:
+            for t in (l if isinstance(l, tuple) else (l,)):
+                n += t.numel() * t.element_size()
+        return n

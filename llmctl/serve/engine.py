@@ -84,6 +84,14 @@ class InferenceEngine:
         self.max_model_len = max_model_len or cfg.max_position_embeddings
         self.block_size = block_size
         self.max_blocks_per_seq = (self.max_model_len + block_size - 1) // block_size
+        # a model of another family (llmctl.models.registry) whose layers mix differently: it runs its
+        # own layers over the step's packed tokens (model.step) against a HybridCache; scheduling,
+        # block tables, state slots, batching and sampling stay the engine's
+        self.hybrid = bool(getattr(self.model, "is_hybrid", False))
+        if self.hybrid:
+            self._init_hybrid(max_batch_size, max_batch_tokens, kv_cache_fraction, num_kv_blocks, scheduler,
+                              prefix_caching, kv_cache_dtype, weight_dtype, seed)
+            return
         # decode projection weights: the model's ("auto"), or an fp8 (OCP e4m3fn) copy with fp32 row
         # scales ("fp8", W8A16) that the fused decode path streams instead (half the bytes of the
         # HBM-bound decode GEMMs); prefill keeps the bf16 weights.  Made before the KV cache is sized.
@@ -139,6 +147,135 @@ class InferenceEngine:
         self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "graph_replays": 0}
         log.info("engine: %s on %s, %d KV blocks x %d tokens (%.1f GB)", cfg.name, self.device, num_kv_blocks,
                  block_size, self.kv_cache.nbytes / 1e9)
+
+    def _init_hybrid(self, max_batch_size, max_batch_tokens, kv_cache_fraction, num_kv_blocks, scheduler,
+                     prefix_caching, kv_cache_dtype, weight_dtype, seed) -> None:
+        from .block_manager import HybridCache
+
+        if self.tp > 1:
+            raise NotImplementedError("hybrid-mixer models serve at TP = 1")
+        if kv_cache_dtype not in ("auto", "model") or weight_dtype not in ("auto", "model"):
+            raise ValueError("hybrid-mixer models keep their cache and weights in the model dtype")
+        self._w8 = self._w8_head = self._nf = None
+        self.weight_dtype, self.kv_dtype, self.rope = "auto", self.dtype, None
+        kinds = []
+        for layer in self.model.layers:
+            m = layer.mixer
+            kinds.append(("latent", m.cache_row) if m.cache_kind == "latent" else ("state", m.state_shapes()))
+        bs = self.block_size
+        if num_kv_blocks is None:
+            if self.device.type == "cuda":
+                torch.cuda.synchronize()
+                free, _ = torch.cuda.mem_get_info(self.device)
+                budget = free * kv_cache_fraction
+            else:
+                budget = 256 * 2 ** 20
+            per = HybridCache.bytes_per_block(kinds, bs, torch.tensor([], dtype=self.dtype).element_size())
+            num_kv_blocks = min(max(int(budget // per), 1), 1 << 20)
+        self.kv_cache = HybridCache(kinds, num_kv_blocks, bs, max_batch_size, self.dtype, self.device)
+        self.kv = make_kv_manager(num_kv_blocks, bs)
+        # a re-attached prefix would skip the tokens that build the recurrent state
+        self.prefix_cache = PrefixCache(self.kv, bs) if prefix_caching and not self.kv_cache.has_state else None
+        self.scheduler = ContinuousBatchScheduler(self.kv, max_batch_size, max_batch_tokens, self.max_model_len,
+                                                  scheduler, bs, prefix_cache=self.prefix_cache,
+                                                  state_slots=self.kv_cache.slots)
+        self.max_batch_size = max_batch_size
+        self.use_graphs = False  # routed experts size their segments on the host
+        self._graphs = {}
+        self._np_rng = np.random.default_rng(seed)
+        self._pending = None
+        self._last_toks = None
+        self.stats = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "graph_replays": 0}
+        log.info("engine: %s on %s, %d cache blocks x %d tokens, %d state slots (%.3f GB)", self.cfg.name, self.device,
+                 num_kv_blocks, bs, max_batch_size, self.kv_cache.nbytes / 1e9)
+
+    def _state_of(self, seqs) -> List[int]:
+        sl = self.kv_cache.slots
+        return [sl.slot(s.seq_id) if sl is not None else 0 for s in seqs]
+
+    @torch.inference_mode()
+    def _hybrid_exec(self, pp: Optional[Dict], dp: Optional[Dict], rows: Optional[List[int]] = None,
+                     trail: Optional[list] = None, count: bool = True) -> torch.Tensor:
+        """One step of a hybrid-mixer model: the prefill plan's packed portions and the decode plan's
+        rows as one token batch through ``model.step``.  Returns logits of ``rows`` (indices into the
+        packed batch; default: the final portions' last rows, then every decode row)."""
+        from llmctl.models.mixers import StepBatch
+
+        use_knobs(self.knobs)
+        d = self.device
+        Tp = len(pp["ids"]) if pp is not None else 0
+        Td = len(dp["ids"]) if dp is not None else 0
+        i32 = lambda a: torch.as_tensor(np.asarray(a, dtype=np.int32)).to(d, non_blocking=True)
+        i64 = lambda a: torch.as_tensor(np.asarray(a, dtype=np.int64)).to(d, non_blocking=True)
+        ids = np.concatenate([np.asarray(pp["ids"], dtype=np.int64) if Tp else np.zeros(0, np.int64),
+                              np.asarray(dp["ids"], dtype=np.int64) if Td else np.zeros(0, np.int64)])
+        pos = np.concatenate([np.asarray(pp["pos"], dtype=np.int32) if Tp else np.zeros(0, np.int32),
+                              np.asarray(dp["positions"], dtype=np.int32) if Td else np.zeros(0, np.int32)])
+        slots = np.concatenate([np.asarray(pp["slots"], dtype=np.int64) if Tp else np.zeros(0, np.int64),
+                                np.asarray(dp["slots"], dtype=np.int64) if Td else np.zeros(0, np.int64)])
+        p_cu = list(pp["cu"]) if Tp else [0]
+        cu = p_cu + [Tp + i + 1 for i in range(Td)]
+        start = ([c - (b - a) for a, b, c in zip(p_cu[:-1], p_cu[1:], pp["ctx"])] if Tp else []) + (
+            list(dp["positions"]) if Td else [])
+        state = (list(pp["state"]) if Tp else []) + (list(dp["state"]) if Td else [])
+        batch = StepBatch(ids=i64(ids), pos=i32(pos), slots=i64(slots), Tp=Tp,
+                          p_cu=i32(p_cu) if Tp else None, p_ctx=i32(pp["ctx"]) if Tp else None,
+                          p_bt=i32(pp["bt"]) if Tp else None, d_ctx=i32(dp["ctx"]) if Td else None,
+                          d_bt=i32(dp["bt"]) if Td else None, cu=i32(cu), start=i32(start), state=i32(state))
+        if rows is None:
+            rows = (list(pp["last"]) if Tp else []) + list(range(Tp, Tp + Td))
+        if count:
+            self.stats["prefill_tokens"] += Tp
+            self.stats["decode_tokens"] += Td
+        if not rows and trail is None:
+            self.model.step(batch, self.kv_cache, rows=i64([]))
+            return torch.empty(0, self.cfg.vocab_size, device=d, dtype=self.dtype)
+        x = self.model.step(batch, self.kv_cache, rows=i64(rows), trail=trail)
+        return self.model.logits(x)
+
+    # ------------------------------------------------------------------ externally driven schedule
+    def open_sequence(self, ids: List[int], request_id: str = "", params: Optional[SamplingParams] = None) -> Sequence:
+        """Admit a sequence outside the queue (the caller dictates what runs in which step)."""
+        seq = Sequence(prompt_ids=list(ids), params=params or SamplingParams(), request_id=request_id)
+        if not self.scheduler.attach(seq):
+            raise RuntimeError("no cache blocks or state slot free for a new sequence")
+        return seq
+
+    def extend_sequence(self, seq: Sequence, ids: List[int]) -> None:
+        if not self.scheduler.extend(seq, list(ids)):
+            raise RuntimeError("no cache blocks free to extend the sequence")
+
+    @torch.inference_mode()
+    def forward_portions(self, portions: List[PrefillChunk], want: List[List[int]], trail: Optional[list] = None):
+        """Run the given portions (sequence, first position, count) as ONE step and return the logits
+        ``[sum(len(w) for w in want), V]`` at the wanted places of each portion (offsets into it), in
+        the order given.  A single token after position 0 runs as a decode row, anything else as a
+        prompt portion; the tokens are marked computed afterwards."""
+        pre = [(i, c) for i, c in enumerate(portions) if not (c.count == 1 and c.start > 0)]
+        dec = [(i, c) for i, c in enumerate(portions) if c.count == 1 and c.start > 0]
+        for _, c in dec:
+            c.seq._decode_slot = int(self.kv.slots(c.seq.seq_id, c.start, 1)[0])
+        pp = self.prefill_plan([c for _, c in pre]) if pre else None
+        dp = None
+        if dec:
+            dp = {"op": "decode", "ids": [c.seq.all_ids[c.start] for _, c in dec], "positions": [c.start for _, c in dec],
+                  "slots": [c.seq._decode_slot for _, c in dec], "ctx": [c.start + 1 for _, c in dec],
+                  "bt": np.asarray(self.kv.block_tables([c.seq.seq_id for _, c in dec], self.max_blocks_per_seq)),
+                  "state": self._state_of([c.seq for _, c in dec]) if self.hybrid else None}
+        base = {}
+        for j, (i, c) in enumerate(pre):
+            base[i] = pp["cu"][j]
+        Tp = len(pp["ids"]) if pp is not None else 0
+        for j, (i, c) in enumerate(dec):
+            base[i] = Tp + j
+        rows = [base[i] + w for i, ws in enumerate(want) for w in ws]
+        if self.hybrid:
+            logits = self._hybrid_exec(pp, dp, rows=rows, trail=trail)
+        else:
+            raise NotImplementedError("forward_portions: hybrid-mixer models only")
+        for c in portions:
+            self.scheduler.computed(c.seq, c.count)
+        return logits
 
     def _fold_norm_weights(self) -> Optional[List[Tuple[torch.Tensor, torch.Tensor]]]:
         """(W_qkv * w_attn_norm, W_up * w_mlp_norm) per layer, or None when the model does not fit
@@ -286,9 +423,12 @@ class InferenceEngine:
         # own rows, so attention can run as packed-document flash attention (doc_start per token)
         fresh = bool(chunks) and all(c.start == 0 for c in chunks)
         doc = np.repeat(np.asarray(cu[:-1], dtype=np.int32), np.diff(cu)) if fresh else None
-        return {"op": "prefill", "ids": np.asarray(ids, dtype=np.int64), "pos": np.asarray(pos, dtype=np.int32),
+        plan = {"op": "prefill", "ids": np.asarray(ids, dtype=np.int64), "pos": np.asarray(pos, dtype=np.int32),
                 "slots": np.concatenate(slots) if slots else np.zeros(0, dtype=np.int64), "cu": cu, "ctx": ctx,
                 "bt": bt, "last": last, "work": ops.prefill_work_list(cu), "doc": doc}
+        if self.hybrid:
+            plan["state"] = self._state_of([c.seq for c in chunks])
+        return plan
 
     @torch.inference_mode()
     def prefill(self, chunks) -> torch.Tensor:
@@ -300,6 +440,8 @@ class InferenceEngine:
 
     @torch.inference_mode()
     def prefill_exec(self, plan: Dict) -> torch.Tensor:
+        if self.hybrid:
+            return self._hybrid_exec(plan, None)
         use_knobs(self.knobs)
         d = self.device
         T = len(plan["ids"])
@@ -369,6 +511,8 @@ class InferenceEngine:
         kernel.  Returns logits [n_final_chunks + n_decode, V]: the final chunks' rows first, in
         chunk order, then the decode rows (eager: the graph-captured decode step is for
         decode-only steps).  Reference batching: ``llmctl/serve/server.py:89-125, 372-386``."""
+        if self.hybrid:
+            return self._hybrid_exec(plan["prefill"], plan["decode"])
         use_knobs(self.knobs)
         d = self.device
         pp, dp = plan["prefill"], plan["decode"]
@@ -616,9 +760,12 @@ class InferenceEngine:
         self.close()
 
     def decode_plan(self, seqs: List[Sequence]) -> Dict:
-        return {"op": "decode", "ids": [s.last_id for s in seqs], "positions": [s.num_tokens - 1 for s in seqs],
+        plan = {"op": "decode", "ids": [s.last_id for s in seqs], "positions": [s.num_tokens - 1 for s in seqs],
                 "slots": [s._decode_slot for s in seqs], "ctx": [self.kv.num_tokens(s.seq_id) for s in seqs],
                 "bt": np.asarray(self.kv.block_tables([s.seq_id for s in seqs], self.max_blocks_per_seq))}
+        if self.hybrid:
+            plan["state"] = self._state_of(seqs)
+        return plan
 
     @torch.inference_mode()
     def decode(self, seqs: List[Sequence]) -> torch.Tensor:
@@ -627,6 +774,8 @@ class InferenceEngine:
     @torch.inference_mode()
     def decode_exec(self, plan: Dict) -> torch.Tensor:
         use_knobs(self.knobs)
+        if self.hybrid:
+            return self._hybrid_exec(None, plan)
         ids, positions, slots, ctx, bt = plan["ids"], plan["positions"], plan["slots"], plan["ctx"], plan["bt"]
         n = len(ids)
         self.stats["decode_tokens"] += n
@@ -739,18 +888,29 @@ class InferenceEngine:
             return b["toks"]
         d = self.device
         n = len(plan["positions"])
+        if self.hybrid:
+            if cont:  # the previous step's sampled ids (this path reads them back: no captured graph)
+                plan = dict(plan, ids=self._last_toks.tolist())
+            logits = self._hybrid_exec(None, plan, count=False)  # counted by _launch_decode
+            toks = self._sample_plan(logits, plan, n)
+            self._last_toks = toks
+            return toks
         ids = self._last_toks if cont else torch.as_tensor(np.asarray(plan["ids"], dtype=np.int64)).to(d)
         logits = self._decode_body(ids, torch.as_tensor(np.asarray(plan["positions"], dtype=np.int32)).to(d),
                                    torch.as_tensor(np.asarray(plan["slots"], dtype=np.int64)).to(d),
                                    torch.from_numpy(np.asarray(plan["bt"])).to(d),
                                    torch.as_tensor(np.asarray(plan["ctx"], dtype=np.int32)).to(d))
+        toks = self._sample_plan(logits, plan, n)
+        self._last_toks = toks
+        return toks
+
+    def _sample_plan(self, logits, plan: Dict, n: int) -> torch.Tensor:
+        d = self.device
         temp = torch.from_numpy(np.asarray(plan["temp"], dtype=np.float32)).to(d)
         topk = torch.from_numpy(np.asarray(plan["topk"], dtype=np.int32)).to(d)
         topp = torch.from_numpy(np.asarray(plan["topp"], dtype=np.float32)).to(d)
         u = torch.from_numpy(np.asarray(plan["u"], dtype=np.float32)).to(d)
-        toks = ops.sample(logits[:n].contiguous(), temp, topk, topp, u)
-        self._last_toks = toks
-        return toks
+        return ops.sample(logits[:n].contiguous(), temp, topk, topp, u)
 
     def _finalize(self, p: Dict) -> int:
         """Read an in-flight step's tokens (the one host sync of the pipeline) and append them."""
@@ -790,6 +950,8 @@ class InferenceEngine:
         plan = {"positions": [s.num_tokens for s in seqs], "slots": [s._decode_slot for s in seqs],
                 "ctx": [self.kv.num_tokens(s.seq_id) for s in seqs],
                 "bt": np.asarray(self.kv.block_tables([s.seq_id for s in seqs], self.max_blocks_per_seq))}
+        if self.hybrid:
+            plan["state"] = self._state_of(seqs)
         self.stats["async_continued"] = self.stats.get("async_continued", 0) + 1
         return self._launch_decode(seqs, plan, cont=True)
 

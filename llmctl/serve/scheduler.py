@@ -105,8 +105,11 @@ class SchedulerOutput:
 
 class ContinuousBatchScheduler:
     def __init__(self, kv, max_batch_size: int = 8, max_batch_tokens: int = 8192, max_model_len: int = 4096,
-                 policy: str = "dynamic", block_size: int = 16, prefix_cache=None):
+                 policy: str = "dynamic", block_size: int = 16, prefix_cache=None, state_slots=None):
         self.kv = kv
+        # recurrent-state slots (block_manager.StateSlotManager) of models that carry a state per
+        # sequence: one is taken at admission and released with the sequence's blocks
+        self.state_slots = state_slots
         self.prefix_cache = prefix_cache
         self.block_size = block_size
         self.max_batch_size = max_batch_size
@@ -139,6 +142,8 @@ class ContinuousBatchScheduler:
     def _can_admit(self) -> bool:
         if not self.waiting or len(self.running) >= self.max_batch_size:
             return False
+        if self.state_slots is not None and self.state_slots.num_free == 0:
+            return False
         n = self.waiting[0].num_tokens + self.kv_block_size()
         if self.kv.can_allocate(n):
             return True
@@ -166,7 +171,11 @@ class ContinuousBatchScheduler:
         need = self.kv.blocks_needed(n + self.kv_block_size()) - len(prefix)
         if not self._reserve(need, protect=prefix):
             return False
+        if self.state_slots is not None and not self.state_slots.alloc(seq.seq_id):
+            return False
         if not self.kv.add_sequence_shared(seq.seq_id, n, prefix):
+            if self.state_slots is not None:
+                self.state_slots.free(seq.seq_id)
             return False
         seq.num_computed = seq.cached_tokens = len(prefix) * self.block_size
         seq.kv_len = n
@@ -270,6 +279,32 @@ class ContinuousBatchScheduler:
             if table:
                 self.prefix_cache.insert(seq.all_ids, table, seq.num_computed, hashes=seq.block_hashes)
         self.kv.free_sequence(seq.seq_id)
+        if self.state_slots is not None:
+            self.state_slots.free(seq.seq_id)
+
+    # ------------------------------------------------------------------ externally driven sequences
+    def attach(self, seq: Sequence) -> bool:
+        """Admit ``seq`` now, outside the queue, with blocks for exactly its known tokens (a caller that
+        dictates the schedule itself: a trace replay, a test).  False if blocks or state slots are short."""
+        if self.state_slots is not None and not self.state_slots.alloc(seq.seq_id):
+            return False
+        if not self._reserve(self.kv.blocks_needed(seq.num_tokens)) or not self.kv.add_sequence(seq.seq_id,
+                                                                                                 seq.num_tokens):
+            if self.state_slots is not None:
+                self.state_slots.free(seq.seq_id)
+            return False
+        seq.status, seq.num_computed, seq.kv_len = "running", 0, seq.num_tokens
+        self.running.append(seq)
+        return True
+
+    def extend(self, seq: Sequence, ids: List[int]) -> bool:
+        """More known tokens for an attached sequence: cache slots for each of them."""
+        for i, t in enumerate(ids):
+            if self.kv.append_token(seq.seq_id) < 0:
+                return False
+            seq.prompt_ids.append(t)
+            seq.kv_len += 1
+        return True
 
     def finish(self, seq: Sequence, reason: str) -> None:
         seq.status = "finished"
