@@ -45,6 +45,7 @@ class StepBatch:
     cu: torch.Tensor  # int32 [n + 1]
     start: torch.Tensor  # int32 [n]
     state: torch.Tensor  # int32 [n]
+    max_q: int = 0  # the longest prompt portion of the step
 
 
 def _init(t: torch.Tensor, std: float) -> None:
@@ -95,7 +96,7 @@ class LatentAttention(nn.Module):
         outs = []
         if b.Tp:
             outs.append(hops.latent_attention_prefill(qa[:b.Tp], cache, b.p_bt, b.p_cu, b.p_ctx, self.window,
-                                                      self.sink, self.scale, self.rk))
+                                                      self.sink, self.scale, self.rk, b.max_q))
         if T > b.Tp:
             outs.append(hops.latent_attention_decode(qa[b.Tp:], cache, b.d_bt, b.d_ctx, self.window, self.sink,
                                                      self.scale, self.rk))

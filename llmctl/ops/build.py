@@ -1,11 +1,13 @@
-"""Build the in-tree HIP kernel library ``llmctl/ops/_llmctl_hip.so`` for gfx950.
+"""Build the in-tree HIP kernel libraries for gfx950: ``llmctl/ops/_llmctl_hip.so`` (group ``core``:
+``csrc/*``) and ``llmctl/ops/_llmctl_hybrid.so`` (group ``hybrid``: ``csrc/hybrid/*``, the kernels of
+the hybrid sequence mixers, a library of their own so that serving such a model needs only it).
 
 Plain ``hipcc`` invocations (no hipify, no torch JIT cache): every ``csrc/*.hip`` /
 ``csrc/*.cpp`` compiles to an object under ``build/ops`` (rebuilt when the content hash of the
 source, the headers or the flags changes), then one link step produces the shared library next to this file, so it
 travels with the repository snapshot to the GPU box.
 
-    python -m llmctl.ops.build [-j N] [--force] [--arch gfx950]
+    python -m llmctl.ops.build [-j N] [--force] [--arch gfx950] [--group core|hybrid|all]
 """
 
 from __future__ import annotations
@@ -22,6 +24,9 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OUT = HERE / "_llmctl_hip.so"
 BUILD = HERE.parents[1] / "build" / "ops"
+# group -> (source directory, library, object directory)
+GROUPS = {"core": (CSRC, OUT, BUILD),
+          "hybrid": (CSRC / "hybrid", HERE / "_llmctl_hybrid.so", BUILD / "hybrid")}
 
 
 def torch_paths():
@@ -61,13 +66,17 @@ def file_flags(src: Path, flags):
     return flags + FILE_FLAGS.get(src.name, [])
 
 
+def _headers(src: Path):
+    return sorted(list(src.parent.glob("*.h")) + list(src.parent.glob("*.inc")))
+
+
 def _digest(src: Path, flags) -> str:
     """Content key of one object: the source, every csrc header and the compile flags (not
     mtimes: a restored or copied tree can carry stale objects with newer timestamps)."""
     import hashlib
 
     h = hashlib.sha256()
-    for d in [src] + sorted(list(CSRC.glob("*.h")) + list(CSRC.glob("*.inc"))):
+    for d in [src] + _headers(src):
         h.update(d.name.encode())
         h.update(d.read_bytes())
     h.update("\0".join(flags).encode())
@@ -79,10 +88,15 @@ def _needs(src: Path, obj: Path, flags) -> bool:
     return not (obj.exists() and key.exists() and key.read_text() == _digest(src, flags))
 
 
-def build(arch: str = "gfx950", jobs: int = 0, force: bool = False, verbose: bool = True) -> Path:
+def build(arch: str = "gfx950", jobs: int = 0, force: bool = False, verbose: bool = True, group: str = "all") -> Path:
+    if group == "all":
+        for g in GROUPS:
+            out = build(arch, jobs, force, verbose, g)
+        return out
+    CSRC, OUT, BUILD = GROUPS[group]
     BUILD.mkdir(parents=True, exist_ok=True)
     srcs = sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
-    flags = compile_flags(arch)
+    flags = compile_flags(arch) + [f"-I{CSRC}"]
     todo = []
     objs = []
     for s in srcs:
@@ -122,13 +136,22 @@ def build(arch: str = "gfx950", jobs: int = 0, force: bool = False, verbose: boo
     return OUT
 
 
+def ensure_group(group: str) -> Path:
+    """Build ``group``'s library if it is not there (first use in a fresh checkout)."""
+    out = GROUPS[group][1]
+    if not out.exists():
+        build(group=group, verbose=False)
+    return out
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--arch", default=os.environ.get("PYTORCH_ROCM_ARCH", "gfx950").split(";")[0])
     ap.add_argument("-j", "--jobs", type=int, default=0)
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--group", default="all", choices=["all"] + sorted(GROUPS))
     a = ap.parse_args(argv)
-    build(a.arch, a.jobs, a.force)
+    build(a.arch, a.jobs, a.force, group=a.group)
 
 
 if __name__ == "__main__":

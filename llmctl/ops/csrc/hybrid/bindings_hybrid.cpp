@@ -1,0 +1,59 @@
+// Operator schemas and registrations of torch.ops.llmctl_hybrid.* (kernels: the .hip files beside
+// this one; CUDA dispatch key == HIP on ROCm builds of PyTorch).
+#include <torch/library.h>
+#include <ATen/ATen.h>
+
+namespace llmctl_hybrid {
+at::Tensor layernorm_f32(const at::Tensor& x, const at::Tensor& w, const at::Tensor& b, double eps, bool out_bf16);
+void residual_add_(at::Tensor x, const at::Tensor& a, const c10::optional<at::Tensor>& b);
+at::Tensor add_layernorm_f32_(at::Tensor x, const at::Tensor& a, const c10::optional<at::Tensor>& b, const at::Tensor& w,
+                              const at::Tensor& bias, double eps, bool out_bf16);
+at::Tensor rmsnorm_cols(const at::Tensor& x, const at::Tensor& w, double eps, int64_t n, bool out_bf16);
+at::Tensor sigmoid_gate_mul(const at::Tensor& o, const at::Tensor& g);
+at::Tensor swiglu_any(const at::Tensor& gu);
+at::Tensor headnorm_gate(const at::Tensor& o, const at::Tensor& w, const at::Tensor& g, double eps, bool out_bf16);
+void latent_kv_write(const at::Tensor& dkv, const at::Tensor& norm_w, double eps, const at::Tensor& pos, const at::Tensor& inv_freq,
+                     int64_t rot_dims, at::Tensor cache, const at::Tensor& slots);
+at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const at::Tensor& pos, const at::Tensor& inv_freq,
+                             int64_t rot_dims, int64_t dn);
+at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& cu,
+                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q);
+at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx,
+                              int64_t window, const at::Tensor& sink, double scale, int64_t rk);
+at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
+                      const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
+                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start);
+std::tuple<at::Tensor, at::Tensor> group_topk_router(const at::Tensor& logits, int64_t top, int64_t groups, int64_t keep);
+}  // namespace llmctl_hybrid
+
+TORCH_LIBRARY(llmctl_hybrid, m) {
+  m.def("layernorm_f32(Tensor x, Tensor w, Tensor b, float eps, bool out_bf16) -> Tensor");
+  m.def("residual_add_(Tensor(a!) x, Tensor a, Tensor? b) -> ()");
+  m.def("add_layernorm_f32_(Tensor(a!) x, Tensor a, Tensor? b, Tensor w, Tensor bias, float eps, bool out_bf16) -> Tensor");
+  m.def("rmsnorm_cols(Tensor x, Tensor w, float eps, int n, bool out_bf16) -> Tensor");
+  m.def("sigmoid_gate_mul(Tensor o, Tensor g) -> Tensor");
+  m.def("swiglu_any(Tensor gu) -> Tensor");
+  m.def("headnorm_gate(Tensor o, Tensor w, Tensor g, float eps, bool out_bf16) -> Tensor");
+  m.def("latent_kv_write(Tensor dkv, Tensor norm_w, float eps, Tensor pos, Tensor inv_freq, int rot_dims, Tensor(a!) cache, Tensor slots) -> ()");
+  m.def("latent_q_assemble(Tensor q_lat, Tensor q, Tensor pos, Tensor inv_freq, int rot_dims, int dn) -> Tensor");
+  m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor sink, float scale, int rk, int max_q) -> Tensor");
+  m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor sink, float scale, int rk) -> Tensor");
+  m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start) -> Tensor");
+  m.def("group_topk_router(Tensor logits, int top, int groups, int keep) -> (Tensor, Tensor)");
+}
+
+TORCH_LIBRARY_IMPL(llmctl_hybrid, CUDA, m) {
+  m.impl("layernorm_f32", &llmctl_hybrid::layernorm_f32);
+  m.impl("residual_add_", &llmctl_hybrid::residual_add_);
+  m.impl("add_layernorm_f32_", &llmctl_hybrid::add_layernorm_f32_);
+  m.impl("rmsnorm_cols", &llmctl_hybrid::rmsnorm_cols);
+  m.impl("sigmoid_gate_mul", &llmctl_hybrid::sigmoid_gate_mul);
+  m.impl("swiglu_any", &llmctl_hybrid::swiglu_any);
+  m.impl("headnorm_gate", &llmctl_hybrid::headnorm_gate);
+  m.impl("latent_kv_write", &llmctl_hybrid::latent_kv_write);
+  m.impl("latent_q_assemble", &llmctl_hybrid::latent_q_assemble);
+  m.impl("latent_attn_prefill", &llmctl_hybrid::latent_attn_prefill);
+  m.impl("latent_attn_decode", &llmctl_hybrid::latent_attn_decode);
+  m.impl("mlstm_scan", &llmctl_hybrid::mlstm_scan);
+  m.impl("group_topk_router", &llmctl_hybrid::group_topk_router);
+}

@@ -1,0 +1,67 @@
+// Helpers of the hybrid-mixer kernels (latent attention, mLSTM, group-limited router, fp32 residual
+// stream).  Every kernel is generic over its sizes (read from the tensors) and templated on the
+// activation element T = float or bf16; all arithmetic is fp32.  Wave size 64.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <ATen/ATen.h>
+#include <ATen/hip/HIPContext.h>
+#include <c10/core/DeviceGuard.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <cstdint>
+
+#define HYB_CHECK(cond, ...) TORCH_CHECK(cond, "llmctl hybrid: ", __VA_ARGS__)
+
+namespace llmctl_hybrid {
+
+using bf16_t = unsigned short;
+
+__device__ __forceinline__ float ldf(const float* p) { return *p; }
+__device__ __forceinline__ float ldf(const bf16_t* p) { return __uint_as_float(((unsigned)*p) << 16); }
+__device__ __forceinline__ void stf(float* p, float v) { *p = v; }
+__device__ __forceinline__ void stf(bf16_t* p, float v) { *p = __bfloat16_as_ushort(__float2bfloat16(v)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Sum over a block of NW waves; every thread gets the result.  ``red`` holds NW floats; two barriers.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();  // red may still be read from a previous call
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) s += red[i];
+  return s;
+}
+
+inline hipStream_t cur_stream() { return at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+template <typename F>
+inline void dispatch_act(const at::Tensor& t, F&& f) {
+  if (t.scalar_type() == at::kFloat) {
+    f((float*)nullptr);
+  } else {
+    HYB_CHECK(t.scalar_type() == at::kBFloat16, "activations must be fp32 or bf16");
+    f((bf16_t*)nullptr);
+  }
+}
+
+inline void check_rows(const at::Tensor& t, const char* name) {
+  HYB_CHECK(t.is_cuda() && t.dim() == 2 && (t.size(1) == 1 || t.stride(1) == 1), name, ": 2-D GPU tensor with unit column stride");
+}
+
+}  // namespace llmctl_hybrid

@@ -67,10 +67,11 @@ def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims: int, dn: int):
     return ref.latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn)
 
 
-def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int):
-    """Prompt portions: sequence n's query rows ``[cu[n], cu[n+1])`` end at position ``ctx[n]-1``."""
+def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int, max_q: int):
+    """Prompt portions: sequence n's query rows ``[cu[n], cu[n+1])`` end at position ``ctx[n]-1``;
+    ``max_q``: the longest portion (sizes the launch)."""
     if use_native(qa):
-        return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk)
+        return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q)
     return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk)
 
 
