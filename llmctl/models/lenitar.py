@@ -202,8 +202,8 @@ class LenitarLM(nn.Module):
                 put(m.q_norm, W[q + "dq.norm"])
                 put(m.kv_norm, W[q + "dkv.norm"])
                 put(m.w_uq, W[q + "uq"])
-                put(m.w_uk, W[q + "uk"].view(m.H, m.dn, m.rk))
-                put(m.w_uv, W[q + "uv"].view(m.H, m.dv, m.rk))
+                put(m.w_uk.view(m.H * m.dn, m.rk), W[q + "uk"])
+                put(m.w_uv.view(m.H * m.dv, m.rk), W[q + "uv"])
                 put(m.sink, W[q + "sink"])
                 put(m.w_o, W[q + "o"])
             else:

@@ -563,6 +563,8 @@ class TrainingEngine:
                 for h in self.metrics_hooks:
                     h(rec)
             if self.faults:
+                if self.faults.due(s):
+                    ckpt.wait()
                 self.faults.after_step(s)
             if c.eval_steps and s % c.eval_steps == 0:
                 ev = [next(data) for _ in range(c.eval_batches)]

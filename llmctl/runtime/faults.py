@@ -61,6 +61,13 @@ class FaultInjector:
         """True when the loss of (1-based) step ``step`` must be poisoned."""
         return any(f.kind == "nan_grad" and f.step == step for f in self.faults)
 
+    def due(self, step: int) -> bool:
+        """True on EVERY rank when a kill / raise of any rank is scheduled after ``step``: the engine
+        first joins its pending asynchronous checkpoint write, so that an injected fault tests the
+        recovery from the last scheduled checkpoint and not the race with its background commit."""
+        return any(f.step == step and f.kind != "nan_grad" and not (self.marker_dir / f.tag).exists()
+                   for f in self.faults)
+
     def after_step(self, step: int) -> None:
         for f in self.faults:
             if f.step != step or f.kind == "nan_grad":

@@ -1,0 +1,302 @@
+"""Lenitar through the serving engine against the plain whole-sequence implementation in
+``tests/oracles/lenitar_plain.py``: every mechanism alone, whole prompts against token-by-token
+decoding, portions down to two tokens, unequal batches, reused pages and state slots, window edges,
+long decoding, other sizes, and greedy generation through the scheduler.
+
+Each test runs on the CPU path and, marked ``gpu``, on the HIP kernels (fp32 with a tight bound, bf16
+with a loose one)."""
+
+import random
+
+import pytest
+import torch
+
+from tests.models import lenitar_util as U
+from tests.oracles import lenitar_plain as plain
+
+DEVICES = [("cpu", torch.float32, 2e-4),
+           pytest.param(("cuda", torch.float32, 2e-4), marks=pytest.mark.gpu),
+           pytest.param(("cuda", torch.bfloat16, 6e-2), marks=pytest.mark.gpu)]
+
+
+@pytest.fixture(params=DEVICES, ids=lambda p: f"{p[0]}-{str(p[1]).split('.')[-1]}")
+def dev(request):
+    return request.param
+
+
+def tokens(n, vocab, seed):
+    r = random.Random(seed)
+    return [r.randrange(vocab) for _ in range(n)]
+
+
+def check(tmp_path, dev, cfg, requests, steps, seed=0, blocks=64, block_size=4, W=None, max_seqs=4):
+    device, dtype, tol = dev
+    W = {k: v.bfloat16().float() for k, v in (W if W is not None else U.random_weights(cfg, seed)).items()}
+    eng = U.engine(U.write_checkpoint(tmp_path / "ck", cfg, W), device, dtype, blocks, block_size, max_seqs)
+    free0 = eng.kv.num_free_blocks
+    got = U.run_schedule(eng, requests, steps)
+    assert eng.kv.num_free_blocks == free0 and (eng.kv_cache.slots is None or eng.kv_cache.slots.num_free == max_seqs)
+    for rid, toks in requests.items():
+        want, _ = plain.forward(toks, W, cfg)
+        err = U.rel_err(got[rid], want.float())
+        assert err < tol, f"{rid}: {err}"
+    eng.close()
+
+
+def whole(requests):
+    return [[(rid, len(t))] for rid, t in requests.items()]
+
+
+# ------------------------------------------------------------------ each mechanism alone
+def test_latent_attention_alone(tmp_path, dev):
+    cfg = U.config([(U.attn(heads=3, dim=8, rot_dim=6, rot_dims=4, vdim=5, kv_rank=9, q_rank=7, window=6), None)])
+    r = {"a": tokens(23, 50, 1)}
+    check(tmp_path, dev, cfg, r, whole(r))
+
+
+def test_latent_attention_one_head_window_one(tmp_path, dev):
+    # a window of 1 sees only the token itself (and the sink)
+    cfg = U.config([(U.attn(heads=1, dim=4, rot_dim=2, vdim=4, kv_rank=4, q_rank=4, window=1), None)])
+    r = {"a": tokens(9, 50, 2)}
+    check(tmp_path, dev, cfg, r, whole(r))
+
+
+def test_sink_takes_weight(tmp_path, dev):
+    # a large sink swallows most of the softmax mass: leaving it out, or counting it per key, shows
+    cfg = U.config([(U.attn(window=7), None)])
+    W = U.random_weights(cfg, 3)
+    W["l0.mix.sink"] = torch.tensor([6.0, -1.0])
+    r = {"a": tokens(15, 50, 3)}
+    check(tmp_path, dev, cfg, r, whole(r), W=W)
+
+
+def test_mlstm_alone(tmp_path, dev):
+    cfg = U.config([(U.rec(heads=3, dim=5, vdim=7, cap=4.0), None)])
+    r = {"a": tokens(40, 50, 4)}
+    check(tmp_path, dev, cfg, r, whole(r))
+
+
+def test_mlstm_wide_head(tmp_path, dev):
+    # more key rows than one register slab tier and more value columns than one tile
+    cfg = U.config([(U.rec(heads=1, dim=70, vdim=130), None)], width=32)
+    r = {"a": tokens(12, 50, 5)}
+    check(tmp_path, dev, cfg, r, whole(r))
+
+
+@pytest.mark.parametrize("router", [dict(experts=6, top=2, groups=3, keep=2), dict(experts=4, top=1, groups=1, keep=1),
+                                    dict(experts=5, top=3, groups=5, keep=4), dict(experts=8, top=4, groups=2, keep=1)])
+def test_moe_alone(tmp_path, dev, router):
+    # the mixer is a one-token window so that the feed-forward carries the test
+    cfg = U.config([(U.attn(window=1), U.moe(ff=6, **router))])
+    r = {"a": tokens(30, 50, 6)}
+    check(tmp_path, dev, cfg, r, whole(r))
+
+
+def test_router_choice():
+    from llmctl.ops import ref_hybrid
+
+    g = torch.Generator().manual_seed(0)
+    h, w = torch.randn(64, 16, generator=g, dtype=torch.float64), torch.randn(12, 16, generator=g, dtype=torch.float64)
+    for top, groups, keep in [(3, 4, 2), (1, 12, 1), (6, 2, 1), (4, 3, 3)]:
+        want_i, want_w = plain.route(h, w, {"experts": 12, "top": top, "groups": {"count": groups, "keep": keep}})
+        got_i, got_w = ref_hybrid.group_topk_router((h @ w.T).float(), top, groups, keep)
+        assert (got_i.sort(-1).values == want_i.sort(-1).values).all()
+        assert torch.allclose(got_w.sort(-1).values.double(), want_w.sort(-1).values, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_router_choice_gpu():
+    from llmctl.ops import hybrid
+
+    g = torch.Generator().manual_seed(1)
+    h, w = torch.randn(300, 16, generator=g, dtype=torch.float64), torch.randn(12, 16, generator=g, dtype=torch.float64)
+    for top, groups, keep in [(3, 4, 2), (1, 12, 1), (6, 2, 1), (4, 3, 3)]:
+        want_i, want_w = plain.route(h, w, {"experts": 12, "top": top, "groups": {"count": groups, "keep": keep}})
+        got_i, got_w = hybrid.group_topk_router((h @ w.T).float().cuda(), top, groups, keep)
+        assert (got_i.cpu().sort(-1).values == want_i.sort(-1).values).all()
+        assert torch.allclose(got_w.cpu().sort(-1).values.double(), want_w.sort(-1).values, atol=1e-6)
+
+
+# ------------------------------------------------------------------ the whole design, other sizes
+FULL = [(U.rec(), U.moe()), (U.attn(), U.moe(experts=4, top=2, groups=2, keep=1)), (U.attn(heads=1, window=3), None),
+        (U.rec(heads=1, dim=9, vdim=4), U.moe(experts=3, top=3, groups=1, keep=1))]
+
+
+def test_all_layers_whole_prompts(tmp_path, dev):
+    cfg = U.config(FULL)
+    r = {"a": tokens(31, 50, 7), "b": tokens(1, 50, 8), "c": tokens(2, 50, 9)}
+    check(tmp_path, dev, cfg, r, whole(r))
+
+
+def test_layers_of_different_sizes(tmp_path, dev):
+    # no two layers alike; kv_rank above one accumulator tier of the decode kernel
+    cfg = U.config([(U.attn(heads=2, dim=6, rot_dim=2, vdim=9, kv_rank=140, q_rank=5, window=4), U.moe()),
+                    (U.attn(heads=4, dim=4, rot_dim=8, rot_dims=6, vdim=4, kv_rank=8, q_rank=16, window=11), None),
+                    (U.rec(heads=2, dim=3, vdim=3), U.moe(experts=2, top=1, groups=2, keep=1, ff=5))], width=20, vocab=33)
+    r = {"a": tokens(26, 33, 10)}
+    check(tmp_path, dev, cfg, r, [[("a", 20)]] + [[("a", 1)]] * 6)
+
+
+# ------------------------------------------------------------------ decode, portions, batches
+def test_prefill_against_token_by_token(tmp_path, dev):
+    cfg = U.config(FULL)
+    r = {"a": tokens(19, 50, 11)}
+    check(tmp_path, dev, cfg, r, [[("a", 1)]] * 19, block_size=4)
+
+
+@pytest.mark.parametrize("sizes", [[2] * 12, [5, 2, 7, 3, 1, 6], [1, 23], [13, 2, 2, 2, 2, 1, 1, 1]])
+def test_portions(tmp_path, dev, sizes):
+    cfg = U.config(FULL)
+    r = {"a": tokens(sum(sizes), 50, 12)}
+    check(tmp_path, dev, cfg, r, [[("a", s)] for s in sizes], block_size=4)
+
+
+def test_unequal_batch_against_each_alone(tmp_path, dev):
+    cfg = U.config(FULL)
+    r = {"a": tokens(30, 50, 13), "b": tokens(9, 50, 14), "c": tokens(17, 50, 15), "d": tokens(3, 50, 16)}
+    steps = [[("a", 11), ("b", 2)], [("a", 1), ("b", 5), ("c", 9)], [("c", 1), ("a", 1), ("d", 3), ("b", 1)],
+             [("a", 7), ("b", 1), ("c", 1)], [("c", 6), ("a", 1)], [("a", 9)]]
+    check(tmp_path, dev, cfg, r, steps, block_size=4)
+
+
+def test_pages_and_slots_used_again(tmp_path, dev):
+    # a pool of 12 pages of 4 tokens and 2 state slots serves five requests one after another and
+    # interleaved; what a finished request left in its pages and slot must not leak into the next
+    cfg = U.config(FULL)
+    r = {k: tokens(n, 50, 20 + i) for i, (k, n) in enumerate([("a", 22), ("b", 18), ("c", 21), ("d", 9), ("e", 20)])}
+    steps = [[("a", 22)], [("b", 10)], [("b", 8), ("c", 5)], [("c", 16)], [("d", 4), ("e", 3)], [("d", 1), ("e", 1)],
+             [("d", 4), ("e", 16)]]
+    check(tmp_path, dev, cfg, r, steps, blocks=12, block_size=4, max_seqs=2)
+
+
+def test_no_slot_left_is_refused(tmp_path):
+    cfg = U.config(FULL)
+    eng = U.engine(U.write_checkpoint(tmp_path / "ck", cfg, U.random_weights(cfg)), "cpu", max_seqs=1)
+    eng.open_sequence([1, 2, 3])
+    with pytest.raises(RuntimeError):
+        eng.open_sequence([4])
+
+
+def test_long_decoding(tmp_path, dev):
+    cfg = U.config(FULL)
+    r = {"a": tokens(140, 50, 30)}
+    check(tmp_path, dev, cfg, r, [[("a", 6)]] + [[("a", 1)]] * 134, block_size=8)
+
+
+def test_state_carries_far_tokens(tmp_path, dev):
+    # slow forgetting: the first tokens still weigh in the output two hundred tokens later, across
+    # portions and decoded tokens, so a state that is lost or restarted shows
+    cfg = U.config([(U.rec(heads=2, dim=6, vdim=8), None)])
+    W = U.random_weights(cfg, 31, forget_bias=7.0)
+    W["l0.mix.i.b"] = torch.tensor([-2.0, -2.0])
+    W["embed"][7] *= 6.0  # one early token writes a large entry into the memory
+    r = {"a": [7] + tokens(220, 50, 32)}
+    check(tmp_path, dev, cfg, r, [[("a", 50)], [("a", 2)], [("a", 100)]] + [[("a", 1)]] * 69, W=W, block_size=16)
+
+
+# ------------------------------------------------------------------ window edges, page borders, far keys
+def _window_case(device, dtype, window, bs, L, j0, form):
+    """One key row j0 that matches every query (score far above the rest): the output at position i is
+    that row's value exactly when 0 <= i - j0 < window."""
+    from llmctl.ops import hybrid
+
+    g = torch.Generator().manual_seed(5)
+    H, rk, dr = 2, 8, 4
+    R = rk + dr
+    nb = (L + bs - 1) // bs + 3
+    perm = torch.randperm(nb, generator=g)
+    rows = torch.randn(L, R, generator=g) * 0.1
+    u = torch.ones(R) / R ** 0.5
+    rows[j0] = 30.0 * u
+    cache = torch.zeros(nb, bs, R)
+    bt = torch.zeros(1, nb, dtype=torch.int32)
+    for p in range(L):
+        bt[0, p // bs] = perm[p // bs]
+        cache[perm[p // bs], p % bs] = rows[p]
+    q = (u[None, None, :] + 0.01 * torch.randn(L, H, R, generator=g))
+    sink = torch.tensor([0.0, -3.0])
+    d = lambda t: t.to(device)
+    cache_d = d(cache.to(dtype))
+    if form == "prefill":
+        out = hybrid.latent_attention_prefill(d(q.to(dtype)), cache_d, d(bt), d(torch.tensor([0, L], dtype=torch.int32)),
+                                              d(torch.tensor([L], dtype=torch.int32)), window, d(sink), 1.0, rk, L)
+    else:
+        out = torch.cat([hybrid.latent_attention_decode(d(q[i:i + 1].to(dtype)), cache_d, d(bt),
+                                                        d(torch.tensor([i + 1], dtype=torch.int32)), window, d(sink), 1.0, rk)
+                         for i in range(L)])
+    out = out.float().cpu()
+    for i in range(L):
+        seen = 0 <= i - j0 < window
+        close = (out[i] - rows[j0, :rk].to(dtype).float()).abs().max() < 0.05
+        assert bool(close) == seen, (form, window, bs, j0, i)
+
+
+@pytest.mark.parametrize("form", ["prefill", "decode"])
+@pytest.mark.parametrize("window,bs,L,j0", [(5, 4, 20, 3), (5, 4, 20, 4), (8, 8, 40, 7), (8, 8, 40, 8), (70, 16, 200, 15),
+                                            (150, 16, 200, 2), (64, 16, 140, 64), (65, 16, 140, 63), (1, 4, 10, 5)])
+def test_window_edges_and_far_keys(dev, form, window, bs, L, j0):
+    _window_case(dev[0], dev[1], window, bs, L, j0, form)
+
+
+def test_window_passes_over_decoded_tokens(tmp_path, dev):
+    # the prompt ends inside the window of the decoded tokens, then the window leaves it
+    cfg = U.config([(U.attn(window=6), None), (U.attn(heads=1, window=9), U.moe())])
+    r = {"a": tokens(40, 50, 40)}
+    check(tmp_path, dev, cfg, r, [[("a", 14)]] + [[("a", 1)]] * 26, block_size=4)
+
+
+# ------------------------------------------------------------------ the framework's own entry point
+def test_greedy_generation_through_the_scheduler(tmp_path, dev):
+    from llmctl.serve.scheduler import SamplingParams
+
+    device, dtype, _ = dev
+    cfg = U.config(FULL)
+    W = U.random_weights(cfg, 50)
+    path = U.write_checkpoint(tmp_path / "ck", cfg, W)
+    eng = U.engine(path, device, dtype, blocks=40, block_size=4, max_seqs=3, scheduler="dynamic")
+    prompts = [tokens(9, 50, 51), tokens(2, 50, 52), tokens(14, 50, 53), tokens(5, 50, 54), tokens(1, 50, 55)]
+    seqs = eng.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True))
+    slack = 1e-3 if dtype == torch.float32 else 0.15
+    for s in seqs:
+        assert len(s.output_ids) == 12
+        logits, _ = plain.forward(s.all_ids[:-1], W, cfg)
+        for k, tok in enumerate(s.output_ids):
+            row = logits[len(s.prompt_ids) - 1 + k]
+            assert row[tok] >= row.max() - slack * float(row.std()), (s.request_id, k)
+    assert eng.kv.num_free_blocks == 40 and eng.kv_cache.slots.num_free == 3
+    eng.close()
+
+
+def test_generation_with_preemption(tmp_path):
+    # too few pages for all requests: the newest is preempted, loses its pages and state slot, and is
+    # recomputed; greedy outputs stay those of an engine with room for all
+    from llmctl.serve.scheduler import SamplingParams
+
+    cfg = U.config(FULL)
+    path = U.write_checkpoint(tmp_path / "ck", cfg, U.random_weights(cfg, 60))
+    prompts = [tokens(6, 50, 61 + i) for i in range(4)]
+    p = SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True)
+    tight = U.engine(path, "cpu", blocks=10, block_size=4, max_seqs=4).generate(prompts, p)
+    roomy = U.engine(path, "cpu", blocks=64, block_size=4, max_seqs=1).generate(prompts, p)
+    assert sum(s.preemptions for s in tight) > 0
+    assert [s.output_ids for s in tight] == [s.output_ids for s in roomy]
+
+
+def test_checkpoint_names_round_trip(tmp_path):
+    from llmctl.models import get_model_config
+    from llmctl.models.lenitar import LenitarLM
+
+    cfg = U.config(FULL)
+    W = U.random_weights(cfg, 70)
+    path = U.write_checkpoint(tmp_path / "ck", cfg, W)
+    c = get_model_config(path)
+    m = LenitarLM(c, dtype=torch.float32)
+    m.load_named(W)
+    back = m.export_named()
+    assert set(back) == set(W)
+    for k in W:
+        assert torch.equal(back[k].float(), W[k]), k
+    bad = dict(W)
+    bad["l1.mix.uk"] = bad["l1.mix.uk"][:-1]
+    with pytest.raises(ValueError):
+        m.load_named(bad)
