@@ -57,11 +57,25 @@ def parse():
     ap.add_argument("--device", default="auto")
     ap.add_argument("--backend", default="auto", help="auto (RCCL on GPU, gloo on CPU) | nccl | gloo")
     ap.add_argument("--json-out", default=None)
+    ap.add_argument("--hybrid-compare", default=None, metavar="SIZES",
+                    help="instead of the training benchmark: serving prefill / decode throughput of Lenitar "
+                         "configurations beside the routed-expert transformer at equal size (comma-separated "
+                         "sizes of llmctl.benchmarks.hybrid.SIZES, or 'all'); one JSON line per size")
     return ap.parse_args()
+
+
+def hybrid_compare(args) -> None:
+    from llmctl.benchmarks import hybrid
+
+    names = sorted(hybrid.SIZES) if args.hybrid_compare == "all" else args.hybrid_compare.split(",")
+    for row in hybrid.run(names, device=args.device, steps=args.steps, warmup=args.warmup):
+        print(json.dumps(row), flush=True)
 
 
 def main():
     args = parse()
+    if args.hybrid_compare:
+        return hybrid_compare(args)
     import torch
     import torch.distributed as dist
 

@@ -1,0 +1,114 @@
+"""Serving throughput of a Lenitar configuration beside the closest existing model (the routed-expert
+transformer: softmax attention + top-k SwiGLU experts) at equal width, depth, heads and experts.
+
+Both run through the same engine calls: one prompt portion per sequence (``InferenceEngine.prefill``)
+and then one-token decode steps of the whole batch (``InferenceEngine.decode``); random weights,
+synthetic tokens.  Reported: prefill tokens/s (one prompt of ``prompt`` tokens) and decode tokens/s
+(``batch`` sequences at that context).
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Dict, List
+
+import torch
+
+SIZES = {
+    "tiny": dict(width=128, layers=4, heads=4, experts=4, top=2, ff=64, window=32, prompt=64, batch=2),
+    # name: width, layers, heads, experts, top, expert ff, window, prompt, decode batch
+    "small": dict(width=1024, layers=4, heads=8, experts=8, top=2, ff=512, window=512, prompt=2048, batch=16),
+    "medium": dict(width=2048, layers=4, heads=16, experts=8, top=2, ff=1024, window=1024, prompt=2048, batch=16),
+    "large": dict(width=4096, layers=4, heads=32, experts=8, top=2, ff=2048, window=1024, prompt=4096, batch=16),
+}
+
+
+def _configs(s: Dict):
+    from llmctl.models.config import ModelConfig
+    from llmctl.models.lenitar import lenitar_template
+
+    hy = lenitar_template(width=s["width"], layers=s["layers"], heads=s["heads"], vocab=32000, every=4,
+                          experts=s["experts"], top=s["top"], groups=2, keep=1, ff=s["ff"], window=s["window"])
+    hy.max_position_embeddings = s["prompt"] + 256
+    tr = ModelConfig(name=f"moe-w{s['width']}-l{s['layers']}", layers=s["layers"], hidden=s["width"], ffn=s["ff"],
+                     heads=s["heads"], vocab_size=32000, max_position_embeddings=s["prompt"] + 256,
+                     num_experts=s["experts"], experts_per_token=s["top"], moe_ffn=s["ff"])
+    return hy, tr
+
+
+def _engine(cfg, device, prompt, batch):
+    import json
+    import tempfile
+    from pathlib import Path
+
+    from llmctl.serve.engine import InferenceEngine
+
+    d = Path(tempfile.mkdtemp(prefix="llmctl_bench_"))
+    (d / "m.json").write_text(json.dumps(cfg.to_dict()))
+    bs = 16
+    blocks = (batch + 1) * ((prompt + 256 + bs - 1) // bs)
+    return InferenceEngine(str(d / "m.json"), device=device, max_batch_size=batch, max_batch_tokens=1 << 30,
+                           max_model_len=prompt + 256, block_size=bs, num_kv_blocks=blocks, use_graphs=False,
+                           prefix_caching=False)
+
+
+def _measure(eng, prompt: int, batch: int, steps: int, warmup: int) -> Dict[str, float]:
+    from llmctl.serve.scheduler import PrefillChunk
+
+    dev = eng.device
+    g = torch.Generator().manual_seed(0)
+    V = eng.cfg.vocab_size
+
+    def sync():
+        if dev.type == "cuda":
+            torch.cuda.synchronize()
+
+    # prefill: one prompt per call
+    times = []
+    for i in range(warmup + steps):
+        seq = eng.open_sequence(torch.randint(0, V, (prompt,), generator=g).tolist())
+        sync()
+        t0 = time.perf_counter()
+        eng.prefill([PrefillChunk(seq, 0, prompt)])
+        sync()
+        times.append(time.perf_counter() - t0)
+        eng.scheduler.computed(seq, prompt)
+        eng.scheduler.finish(seq, "stop")
+    pre = sorted(times[warmup:])[len(times[warmup:]) // 2]
+    # decode: ``batch`` sequences at context ``prompt``
+    seqs = [eng.open_sequence(torch.randint(0, V, (prompt,), generator=g).tolist()) for _ in range(batch)]
+    for s in seqs:
+        eng.prefill([PrefillChunk(s, 0, prompt)])
+        eng.scheduler.computed(s, prompt)
+    times = []
+    for i in range(warmup + steps):
+        for s in seqs:
+            eng.scheduler.extend(s, [int(torch.randint(0, V, (1,), generator=g))])
+            s._decode_slot = int(eng.kv.slots(s.seq_id, s.num_tokens - 1, 1)[0])
+        sync()
+        t0 = time.perf_counter()
+        eng.decode(seqs)
+        sync()
+        times.append(time.perf_counter() - t0)
+        for s in seqs:
+            eng.scheduler.computed(s, 1)
+    dec = sorted(times[warmup:])[len(times[warmup:]) // 2]
+    for s in seqs:
+        eng.scheduler.finish(s, "stop")
+    return {"prefill_ms": round(pre * 1e3, 3), "prefill_tok_s": round(prompt / pre, 1),
+            "decode_ms": round(dec * 1e3, 3), "decode_tok_s": round(batch / dec, 1)}
+
+
+def run(sizes: List[str], device: str = "auto", steps: int = 5, warmup: int = 2) -> List[Dict]:
+    out = []
+    for name in sizes:
+        s = SIZES[name]
+        hy, tr = _configs(s)
+        row = {"size": name, **{k: s[k] for k in ("width", "layers", "heads", "experts", "top", "ff", "window", "prompt", "batch")}}
+        for label, cfg in (("lenitar", hy), ("moe_transformer", tr)):
+            eng = _engine(cfg, device, s["prompt"], s["batch"])
+            row[label] = _measure(eng, s["prompt"], s["batch"], steps, warmup)
+            row[label]["params_m"] = round(sum(p.numel() for p in eng.model.parameters()) / 1e6, 1)
+            eng.close()
+        out.append(row)
+    return out
