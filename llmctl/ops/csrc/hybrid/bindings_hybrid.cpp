@@ -17,9 +17,9 @@ void latent_kv_write(const at::Tensor& dkv, const at::Tensor& norm_w, double eps
 at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const at::Tensor& pos, const at::Tensor& inv_freq,
                              int64_t rot_dims, int64_t dn);
 at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& cu,
-                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q);
+                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q, bool mfma);
 at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx,
-                              int64_t window, const at::Tensor& sink, double scale, int64_t rk);
+                              int64_t window, const at::Tensor& sink, double scale, int64_t rk, bool mfma);
 at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
                       const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
                       const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start);
@@ -36,8 +36,8 @@ TORCH_LIBRARY(llmctl_hybrid, m) {
   m.def("headnorm_gate(Tensor o, Tensor w, Tensor g, float eps, bool out_bf16) -> Tensor");
   m.def("latent_kv_write(Tensor dkv, Tensor norm_w, float eps, Tensor pos, Tensor inv_freq, int rot_dims, Tensor(a!) cache, Tensor slots) -> ()");
   m.def("latent_q_assemble(Tensor q_lat, Tensor q, Tensor pos, Tensor inv_freq, int rot_dims, int dn) -> Tensor");
-  m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor sink, float scale, int rk, int max_q) -> Tensor");
-  m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor sink, float scale, int rk) -> Tensor");
+  m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor sink, float scale, int rk, int max_q, bool mfma=True) -> Tensor");
+  m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor sink, float scale, int rk, bool mfma=True) -> Tensor");
   m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start) -> Tensor");
   m.def("group_topk_router(Tensor logits, int top, int groups, int keep) -> (Tensor, Tensor)");
 }

@@ -213,6 +213,11 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
   }
 }
 
+// latent_attn_mfma.hip: the matrix-core form for bf16 shapes that fit it
+bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk);
+void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor* cu, const at::Tensor& ctx,
+                      int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out);
+
 // ------------------------------------------------------------------------------------------ host
 static void check_cache(const at::Tensor& cache, const at::Tensor& like, int64_t R) {
   HYB_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R && cache.scalar_type() == like.scalar_type(),
@@ -265,7 +270,8 @@ at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const
 }
 
 at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& cu,
-                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q) {
+                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q,
+                               bool mfma) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [T, H, R]");
   const int64_t T = qa.size(0), H = qa.size(1), R = qa.size(2);
   check_cache(cache, qa, R);
@@ -280,6 +286,10 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({T, H, rk}, qa.options());
   if (T == 0 || ns == 0) return out;
+  if (mfma && latent_attn_mfma_ok(qa, rk)) {
+    latent_attn_mfma(qa, cache, bt, &cu, ctx, window, sink, scale, rk, max_q, out);
+    return out;
+  }
   const int VT = rk <= 32 ? 32 : (rk <= 64 ? 64 : 128);
   const int nvt = (int)((rk + VT - 1) / VT);
   HYB_CHECK(H * nvt <= 65535 && ns <= 65535, "grid too large");
@@ -301,7 +311,7 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
 }
 
 at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx,
-                              int64_t window, const at::Tensor& sink, double scale, int64_t rk) {
+                              int64_t window, const at::Tensor& sink, double scale, int64_t rk, bool mfma) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [n, H, R]");
   const int64_t ns = qa.size(0), H = qa.size(1), R = qa.size(2);
   check_cache(cache, qa, R);
@@ -309,10 +319,15 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
   check_i32(ctx, "ctx");
   HYB_CHECK(bt.dim() == 2 && bt.size(0) == ns && ctx.numel() == ns, "block tables [n, max_blocks], ctx [n]");
   HYB_CHECK(sink.is_cuda() && sink.scalar_type() == at::kFloat && sink.is_contiguous() && sink.numel() == H, "sink: fp32 [H]");
-  HYB_CHECK(rk >= 1 && rk <= R && rk <= 512 && window >= 1, "rank <= min(R, 512), window >= 1");
+  HYB_CHECK(rk >= 1 && rk <= R && window >= 1, "rank <= R, window >= 1");
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({ns, H, rk}, qa.options());
   if (ns == 0) return out;
+  if (mfma && latent_attn_mfma_ok(qa, rk)) {
+    latent_attn_mfma(qa, cache, bt, nullptr, ctx, window, sink, scale, rk, 1, out);
+    return out;
+  }
+  HYB_CHECK(rk <= 512, "generic decode kernel: rank <= 512");
   const int64_t Rp = R + (R & 1);  // keeps the int64 array 8-byte aligned
   const size_t lds = (size_t)(Rp + 256) * 4 + 256 * 8 + 8 * 4 + (size_t)4 * rk * 4;
   HYB_CHECK(lds <= 64 * 1024 && H <= 65535, "rank + rot too wide");

@@ -1,0 +1,242 @@
+// Latent attention on the matrix cores (bf16; MFMA 32x32x16), prompt portions and decode rows alike.
+//
+// The cache row [latent | rotary key] of width R is key and, in its first ``rank`` entries, value; the
+// queries come in the same layout (see latent_attn.hip).  This is the flash-attention forward of the
+// framework's paged prefill kernel re-cut for that layout:
+//   * a workgroup (4 waves) owns 128 query rows = TB tokens x HB heads of one sequence (HB = 1 for
+//     long portions, = the head count for decode rows and short portions, where the heads of a token
+//     fill the tile and share every key row);
+//   * tiles of 64 keys, gathered through the block table into LDS once per workgroup: a "row image"
+//     of all of R (in column blocks of 128) for S^T = K Q^T, and a "transposed-read image" of the
+//     column blocks that hold this workgroup's value columns for O^T += V^T P^T;
+//   * Q fragments stay in registers for the whole key loop; softmax is lane-local (query on the lane),
+//     exp2 domain, deferred rescale; the sink starts the running maximum and the denominator;
+//   * the key loop runs only over the tiles that the rows' windows touch.
+// Value columns beyond 256 go to further workgroups (blockIdx.z), which recompute the scores.
+// Shapes it takes: R and rank multiples of 8, R <= 640; anything else runs the generic kernels.
+#include "attn_common.h"
+#include "hybrid_common.h"
+
+namespace llmctl_hybrid {
+using namespace llmctl::attn;
+
+namespace {
+constexpr int LKB = 64;         // keys per tile
+constexpr int LROWB = 256;      // bytes of one row of a 128-column block image
+constexpr int LIMG = LKB * LROWB;
+constexpr float kRescaleTh = 8.f;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct LArgs {
+  const unsigned short* qa;
+  const unsigned short* cache;
+  unsigned short* out;
+  const int* bt;
+  const int* cu;   // nullptr: one query row per sequence (decode)
+  const int* ctx;
+  const float* sink;
+  int H, R, rk, bs, maxb, window, HB, nvt;
+  float scale_log2;
+};
+
+template <int NCB, int NDB>
+__global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
+  constexpr int NKS = NCB * 8;
+  constexpr int NTB = (NDB + 3) / 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* Ks = smem;
+  unsigned char* Vs = smem + NCB * LIMG;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, hh = lane >> 5;
+  const int n = blockIdx.y;
+  const int hg = blockIdx.z / a.nvt, v0 = (blockIdx.z % a.nvt) * (NDB * 32);
+  const int q_begin = a.cu ? a.cu[n] : n;
+  const int qlen = a.cu ? a.cu[n + 1] - q_begin : 1;
+  const int HB = a.HB, TB = 128 / HB;
+  const int tok0 = blockIdx.x * TB;
+  if (tok0 >= qlen) return;
+  const int ctx = a.ctx[n];
+  const int pos0 = ctx - qlen;
+  const int row = wave * 32 + r;
+  const int my_tok = tok0 + row / HB, my_head = hg * HB + row % HB;
+  const bool valid = my_tok < qlen && my_head < a.H;
+  const int tokc = min(my_tok, qlen - 1), headc = min(my_head, a.H - 1);
+  const int my_pos = pos0 + tokc;
+  const int* btn = a.bt + (long)n * a.maxb;
+
+  bf16x8_t qf[NKS];
+  {
+    const unsigned short* Qp = a.qa + ((long)(q_begin + tokc) * a.H + headc) * a.R;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int col = ks * 16 + 8 * hh;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (col < a.R) v = gload16(Qp + col);
+      qf[ks] = __builtin_bit_cast(bf16x8_t, v);
+    }
+  }
+  f32x16 o[NDB];
+#pragma unroll
+  for (int d = 0; d < NDB; ++d)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
+  float m_i = a.sink[headc] * kLog2e, l_i = 1.0f;  // the sink: one unit of mass at its own logit
+
+  const int first_pos = pos0 + tok0, last_pos = pos0 + min(tok0 + TB, qlen) - 1;
+  const int t_lo = max(0, first_pos - a.window + 1) / LKB, t_hi = last_pos / LKB + 1;
+  // this wave's rows: positions [w_first, w_last]
+  const int w_first = pos0 + min(tok0 + (wave * 32) / HB, qlen - 1);
+  const int w_last = pos0 + min(tok0 + (wave * 32 + 31) / HB, qlen - 1);
+  const bool wave_live = tok0 + (wave * 32) / HB < qlen && hg * HB + (HB >= 32 ? (wave * 32) % HB : 0) < a.H;
+
+  constexpr int CPT = NCB * 16;  // 16-byte chunks of one key row (padded R)
+  for (int t = t_lo; t < t_hi; ++t) {
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < NCB * 4; ++it) {
+      const int c = tid + 256 * it;
+      const int krow = c / CPT, ch = c % CPT;
+      const int key = t * LKB + krow, col = ch * 8;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (key < ctx && col < a.R) {
+        const long slot = (long)btn[key / a.bs] * a.bs + key % a.bs;
+        v = gload16(a.cache + slot * a.R + col);
+      }
+      const int cb = ch >> 4, chb = ch & 15;
+      *reinterpret_cast<uint4*>(Ks + cb * LIMG + row_off<128>(krow, chb)) = v;
+      const int tb = cb - v0 / 128;
+      if (tb >= 0 && tb < NTB) *reinterpret_cast<uint4*>(Vs + tb * LIMG + tr_off<128>(krow, chb)) = v;
+    }
+    __syncthreads();
+    const int kv0 = t * LKB;
+    if (!wave_live || kv0 > w_last || kv0 + LKB - 1 < w_first - a.window + 1) continue;
+
+    f32x16 s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const bf16x8_t kf = lds_read_b128(Ks + (ks >> 3) * LIMG, row_off<128>(kb * 32 + r, (2 * ks + hh) & 15));
+        s[kb] = mfma32(kf, qf[ks], s[kb]);
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float x = s[kb][i] * a.scale_log2;
+        const int key = kv0 + kb * 32 + acc_row(i, hh);
+        if (!valid || key > my_pos || key <= my_pos - a.window || key >= ctx) x = -INFINITY;
+        s[kb][i] = x;
+        mx = fmaxf(mx, x);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const bool grow = __builtin_amdgcn_ballot_w64(mx > m_i + kRescaleTh) != 0;
+    const float m_new = grow ? fmaxf(m_i, mx) : m_i;
+    float rs = 0.f;
+    bf16x8_t pb[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      float p[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        p[i] = fast_exp2(s[kb][i] - m_new);
+        rs += p[i];
+      }
+      pb[kb][0] = to_bf16x8(p);
+      pb[kb][1] = to_bf16x8(p + 8);
+    }
+    rs += __shfl_xor(rs, 32);
+    if (grow) {
+      const float alpha = fast_exp2(m_i - m_new);
+      l_i *= alpha;
+#pragma unroll
+      for (int d = 0; d < NDB; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+    }
+    l_i += rs;
+    m_i = m_new;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int d = 0; d < NDB; ++d) {
+          const bf16x8_t vf = tr_frag<128>(Vs + (d >> 2) * LIMG, kb * 32 + 16 * st, (d & 3) * 32, lane);
+          o[d] = mfma32(vf, pb[kb][st], o[d]);
+        }
+  }
+
+  if (valid) {
+    const float inv = 1.f / l_i;
+    unsigned short* Op = a.out + ((long)(q_begin + my_tok) * a.H + my_head) * a.rk;
+#pragma unroll
+    for (int d = 0; d < NDB; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int col = v0 + d * 32 + 8 * g + 4 * hh;
+        if (col < a.rk) {
+          unsigned short w4[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) w4[j] = __bfloat16_as_ushort(__float2bfloat16(o[d][4 * g + j] * inv));
+          *reinterpret_cast<uint2*>(Op + col) =
+              make_uint2((unsigned)w4[0] | ((unsigned)w4[1] << 16), (unsigned)w4[2] | ((unsigned)w4[3] << 16));
+        }
+      }
+  }
+}
+
+template <int NCB>
+void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
+  auto go = [&](auto kern, int NDBv) {
+    const size_t lds = (size_t)(NCB + (NDBv + 3) / 4) * LIMG;
+    HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
+    kern<<<grid, 256, lds, st>>>(a);
+  };
+  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2>, 2);
+  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4>, 4);
+  else go(latent_attn_mfma_kernel<NCB, 8>, 8);
+}
+}  // namespace
+
+bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk) {
+  const int64_t R = qa.size(2);
+  return qa.scalar_type() == at::kBFloat16 && R % 8 == 0 && rk % 8 == 0 && R <= 640 && qa.size(1) >= 1;
+}
+
+// cu: undefined tensor = one row per sequence
+void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor* cu, const at::Tensor& ctx,
+                      int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out) {
+  const int64_t H = qa.size(1), R = qa.size(2), ns = ctx.numel();
+  const int ncb = (int)((R + 127) / 128);
+  const int ndb = rk <= 64 ? 2 : (rk <= 128 ? 4 : 8);
+  const int nvt = (int)((rk + ndb * 32 - 1) / (ndb * 32));
+  int HB = 1;
+  if (max_q < 64) {
+    while (HB < H && HB < 128) HB *= 2;
+  }
+  const int TB = 128 / HB;
+  const int hgroups = (int)((H + HB - 1) / HB);
+  HYB_CHECK(ns <= 65535 && hgroups * nvt <= 65535, "grid too large");
+  LArgs a{reinterpret_cast<const unsigned short*>(qa.data_ptr()), reinterpret_cast<const unsigned short*>(cache.data_ptr()),
+          reinterpret_cast<unsigned short*>(out.data_ptr()), bt.data_ptr<int>(), cu ? cu->data_ptr<int>() : nullptr, ctx.data_ptr<int>(),
+          sink.data_ptr<float>(), (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
+          (float)(scale * 1.4426950408889634)};
+  dim3 grid((unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
+  hipStream_t st = cur_stream();
+  switch (ncb) {
+    case 1: launch_ncb<1>(a, ndb, grid, st); break;
+    case 2: launch_ncb<2>(a, ndb, grid, st); break;
+    case 3: launch_ncb<3>(a, ndb, grid, st); break;
+    case 4: launch_ncb<4>(a, ndb, grid, st); break;
+    default: launch_ncb<5>(a, ndb, grid, st); break;
+  }
+}
+
+}  // namespace llmctl_hybrid

@@ -67,18 +67,20 @@ def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims: int, dn: int):
     return ref.latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn)
 
 
-def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int, max_q: int):
+def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int, max_q: int,
+                             mfma: bool = True):
     """Prompt portions: sequence n's query rows ``[cu[n], cu[n+1])`` end at position ``ctx[n]-1``;
-    ``max_q``: the longest portion (sizes the launch)."""
+    ``max_q``: the longest portion (sizes the launch).  bf16 shapes that fit run on the matrix cores
+    (``mfma=False`` forces the generic fp32-SIMT kernel, which also serves fp32)."""
     if use_native(qa):
-        return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q)
+        return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q, mfma)
     return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk)
 
 
-def latent_attention_decode(qa, cache, bt, ctx, window: int, sink, scale: float, rk: int):
+def latent_attention_decode(qa, cache, bt, ctx, window: int, sink, scale: float, rk: int, mfma: bool = True):
     """One query row per sequence, at position ``ctx[n] - 1``."""
     if use_native(qa):
-        return native_hybrid().latent_attn_decode(qa, cache, bt, ctx, window, sink, scale, rk)
+        return native_hybrid().latent_attn_decode(qa, cache, bt, ctx, window, sink, scale, rk, mfma)
     cu = torch.arange(qa.shape[0] + 1, dtype=torch.int32)
     return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk)
 

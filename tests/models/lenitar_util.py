@@ -14,7 +14,7 @@ from llmctl.serve.engine import InferenceEngine
 from llmctl.serve.scheduler import PrefillChunk
 
 
-def attn(heads=2, dim=8, rot_dim=4, vdim=6, kv_rank=12, q_rank=10, window=5, base=100.0, rot_dims=None, scale=None):
+def attn(heads=2, dim=8, rot_dim=8, vdim=6, kv_rank=16, q_rank=10, window=5, base=100.0, rot_dims=None, scale=None):
     return {"type": "latent_attention",
             "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
                       "rot": {"base": base, "dims": rot_dims if rot_dims is not None else rot_dim},

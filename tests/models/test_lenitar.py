@@ -195,13 +195,13 @@ def test_state_carries_far_tokens(tmp_path, dev):
 
 
 # ------------------------------------------------------------------ window edges, page borders, far keys
-def _window_case(device, dtype, window, bs, L, j0, form):
+def _window_case(device, dtype, window, bs, L, j0, form, mfma=True):
     """One key row j0 that matches every query (score far above the rest): the output at position i is
     that row's value exactly when 0 <= i - j0 < window."""
     from llmctl.ops import hybrid
 
     g = torch.Generator().manual_seed(5)
-    H, rk, dr = 2, 8, 4
+    H, rk, dr = 2, 8, 8
     R = rk + dr
     nb = (L + bs - 1) // bs + 3
     perm = torch.randperm(nb, generator=g)
@@ -219,10 +219,10 @@ def _window_case(device, dtype, window, bs, L, j0, form):
     cache_d = d(cache.to(dtype))
     if form == "prefill":
         out = hybrid.latent_attention_prefill(d(q.to(dtype)), cache_d, d(bt), d(torch.tensor([0, L], dtype=torch.int32)),
-                                              d(torch.tensor([L], dtype=torch.int32)), window, d(sink), 1.0, rk, L)
+                                              d(torch.tensor([L], dtype=torch.int32)), window, d(sink), 1.0, rk, L, mfma)
     else:
         out = torch.cat([hybrid.latent_attention_decode(d(q[i:i + 1].to(dtype)), cache_d, d(bt),
-                                                        d(torch.tensor([i + 1], dtype=torch.int32)), window, d(sink), 1.0, rk)
+                                                        d(torch.tensor([i + 1], dtype=torch.int32)), window, d(sink), 1.0, rk, mfma)
                          for i in range(L)])
     out = out.float().cpu()
     for i in range(L):
@@ -236,6 +236,64 @@ def _window_case(device, dtype, window, bs, L, j0, form):
                                             (150, 16, 200, 2), (64, 16, 140, 64), (65, 16, 140, 63), (1, 4, 10, 5)])
 def test_window_edges_and_far_keys(dev, form, window, bs, L, j0):
     _window_case(dev[0], dev[1], window, bs, L, j0, form)
+    if dev[1] == torch.bfloat16:  # the generic kernel too (bf16 defaults to the matrix-core form)
+        _window_case(dev[0], dev[1], window, bs, L, j0, form, mfma=False)
+
+
+def _direct_attention(qa, rows, qpos, window, sink, scale, rk):
+    """qa [T, H, R], rows [L, R] (one sequence's cache rows in order), qpos [T]."""
+    s = torch.einsum("thr,kr->htk", qa.double(), rows.double()) * scale
+    d = qpos[:, None] - torch.arange(rows.shape[0])[None, :]
+    s = s.masked_fill(~((d >= 0) & (d < window)), float("-inf"))
+    sk = sink.double().view(-1, 1, 1)
+    top = torch.maximum(s.max(-1, keepdim=True).values, sk)
+    e = torch.exp(s - top)
+    p = e / (e.sum(-1, keepdim=True) + torch.exp(sk - top))
+    return torch.einsum("htk,kr->thr", p, rows[:, :rk].double())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,rk,dr,window,bs", [(6, 88, 24, 70, 16), (3, 40, 8, 21, 16), (16, 512, 64, 300, 16),
+                                               (40, 136, 64, 64, 8), (5, 264, 24, 1000, 32)])
+def test_latent_attention_kernels_gpu(H, rk, dr, window, bs):
+    # several sequences: long portions, a two-token portion, a first token, decode rows; both kernel
+    # forms (matrix cores / generic) in bf16 and the generic one in fp32, against the direct formula
+    from llmctl.ops import hybrid
+
+    g = torch.Generator().manual_seed(H)
+    R = rk + dr
+    lens, chunk = [330, 200, 2, 1, 97, 64], [330, 130, 2, 1, 1, 1]
+    nb = sum((L + bs - 1) // bs for L in lens) + 2
+    perm = torch.randperm(nb, generator=g).tolist()
+    bt = torch.zeros(len(lens), max((L + bs - 1) // bs for L in lens), dtype=torch.int32)
+    cache = torch.zeros(nb, bs, R)
+    seq_rows, k = [], 0
+    for i, L in enumerate(lens):
+        rows = (torch.randn(L, R, generator=g) * 0.7).bfloat16().float()
+        seq_rows.append(rows)
+        for j in range((L + bs - 1) // bs):
+            bt[i, j] = perm[k]
+            cache[perm[k], :min(bs, L - j * bs)] = rows[j * bs:(j + 1) * bs]
+            k += 1
+    sink = torch.randn(H, generator=g)
+    scale = R ** -0.5
+    qs = [(torch.randn(c, H, R, generator=g)).bfloat16().float() for c in chunk]
+    want = [_direct_attention(q, rows, torch.arange(L - c, L), window, sink, scale, rk)
+            for q, rows, L, c in zip(qs, seq_rows, lens, chunk)]
+    npre = 3
+    for dtype, mfma, tol in [(torch.bfloat16, True, 2e-2), (torch.bfloat16, False, 2e-2), (torch.float32, False, 2e-5)]:
+        c_d = cache.to(dtype).cuda()
+        cu = torch.tensor([0] + list(torch.tensor(chunk[:npre]).cumsum(0)), dtype=torch.int32).cuda()
+        out_p = hybrid.latent_attention_prefill(torch.cat(qs[:npre]).to(dtype).cuda(), c_d, bt[:npre].cuda(), cu,
+                                                torch.tensor(lens[:npre], dtype=torch.int32).cuda(), window, sink.cuda(),
+                                                scale, rk, max(chunk[:npre]), mfma)
+        out_d = hybrid.latent_attention_decode(torch.cat(qs[npre:]).to(dtype).cuda(), c_d, bt[npre:].contiguous().cuda(),
+                                               torch.tensor(lens[npre:], dtype=torch.int32).cuda(), window, sink.cuda(),
+                                               scale, rk, mfma)
+        got = torch.cat([out_p, out_d]).float().cpu()
+        ref = torch.cat(want).float()
+        err = (got - ref).abs().max() / ref.abs().max()
+        assert err < tol, (dtype, mfma, float(err))
 
 
 def test_window_passes_over_decoded_tokens(tmp_path, dev):
