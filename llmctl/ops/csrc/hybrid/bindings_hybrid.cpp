@@ -22,7 +22,7 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
                               int64_t window, const at::Tensor& sink, double scale, int64_t rk, bool mfma);
 at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
                       const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
-                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start);
+                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab);
 std::tuple<at::Tensor, at::Tensor> group_topk_router(const at::Tensor& logits, int64_t top, int64_t groups, int64_t keep);
 }  // namespace llmctl_hybrid
 
@@ -38,7 +38,7 @@ TORCH_LIBRARY(llmctl_hybrid, m) {
   m.def("latent_q_assemble(Tensor q_lat, Tensor q, Tensor pos, Tensor inv_freq, int rot_dims, int dn) -> Tensor");
   m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor sink, float scale, int rk, int max_q, bool mfma=True) -> Tensor");
   m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor sink, float scale, int rk, bool mfma=True) -> Tensor");
-  m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start) -> Tensor");
+  m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start, bool slab=False) -> Tensor");
   m.def("group_topk_router(Tensor logits, int top, int groups, int keep) -> (Tensor, Tensor)");
 }
 

@@ -3,19 +3,163 @@
 //   i = cap tanh((zi + bi) / cap),   f = logsigmoid(cap tanh((zf + bf) / cap)):
 //   m' = max(f + m, i);  S = e^(f + m - m') S + e^(i - m') k v^T;  n likewise with k alone;
 //   o = S^T q / (max(|n . q|, e^(-m')) + 1e-6),  q already scaled.
-// One block per (sequence, head, tile of 64 value columns): 4 waves split the dk rows into slabs, a
-// lane owns one column of its slab in registers; lane r of a slab also owns n[row r of the slab].
-// Column sums over slabs and n . q go through LDS (two barriers per token, double-buffered).
+// A pre-pass turns the gate pre-activations into i and f for all tokens at once.  The scan has two forms:
+//   * dk <= 128: one wave per (sequence, head, tile of 64 value columns), a lane owns one column of S
+//     (all dk rows in registers); k and q are spread over the lanes and reach the column update as
+//     scalar operands (v_readlane), n is spread over the lanes and n . q is one wave reduction: no LDS
+//     and no barrier in the token loop; the next token's operands are loaded during the current update;
+//   * dk <= 512: one block per (sequence, head, tile): 4 waves split the dk rows into slabs, column
+//     sums over slabs and n . q go through LDS (two barriers per token, double-buffered).
 #include "hybrid_common.h"
+
+#include <type_traits>
 
 namespace llmctl_hybrid {
 
 __device__ __forceinline__ float log_sigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
+// raw [T, 2H] -> (i, f): i = cap tanh((z_i + b_i) / cap), f = logsigmoid(cap tanh((z_f + b_f) / cap))
+__global__ void mlstm_gates_kernel(const float* __restrict__ raw, const float* __restrict__ b_i, const float* __restrict__ b_f,
+                                   float cap, float* __restrict__ out, int64_t T, int H) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * 2 * H) return;
+  const int c = (int)(i % (2 * H));
+  if (c < H) out[i] = cap * tanhf((raw[i] + b_i[c]) / cap);
+  else out[i] = log_sigmoid(cap * tanhf((raw[i] + b_f[c - H]) / cap));
+}
+
+// Sum over the wave on the VALU's data-parallel primitives (quad swaps, half-row and row mirrors), then
+// the four row sums through scalar registers: no LDS round trips.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  v += dpp(v, std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+  v += dpp(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+  v += dpp(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
+  v += dpp(v, std::integral_constant<int, 0x140>{});  // row_mirror
+  auto rl = [](float x, int l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l)); };
+  return (rl(v, 0) + rl(v, 16)) + (rl(v, 32) + rl(v, 48));
+}
+
+// One wave per (sequence, head, 64 value columns); DK = register rows (>= dk), a multiple of 16.
+// k and q of the token go through a wave-private LDS line and come back as broadcast reads.
+template <typename T, int DK>
+__global__ __launch_bounds__(64) void mlstm_scan_wave_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                                             int64_t row_stride, const float* __restrict__ gates, float qscale,
+                                                             float* __restrict__ Sp, float* __restrict__ np, float* __restrict__ mp,
+                                                             const int* __restrict__ slots, const int* __restrict__ cu,
+                                                             const int* __restrict__ start, float* __restrict__ out, int H, int dk,
+                                                             int dv) {
+  constexpr int NR = (DK + 63) / 64;
+  constexpr int DP = NR * 64;
+  __shared__ __attribute__((aligned(16))) float kq[2][2 * DP];
+  const int sq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
+  const int a = cu[sq], b = cu[sq + 1];
+  if (a == b) return;
+  const int lane = threadIdx.x;
+  const int col = v0 + lane;
+  const bool cok = col < dv;
+  const int64_t slot = slots[sq];
+  float* Sb = Sp + (slot * H + h) * (int64_t)dk * dv;
+  float* nb = np + (slot * H + h) * (int64_t)dk;
+  const bool fresh = start[sq] == 0;
+  float S[DK], nr[NR];
+#pragma unroll
+  for (int d = 0; d < DK; ++d) S[d] = (!fresh && cok && d < dk) ? Sb[(int64_t)d * dv + col] : 0.f;
+#pragma unroll
+  for (int i = 0; i < NR; ++i) nr[i] = (!fresh && lane + 64 * i < dk) ? nb[lane + 64 * i] : 0.f;
+  float m = fresh ? 0.f : mp[slot * H + h];
+  // operands of TBATCH tokens are loaded ahead, one batch in flight while the previous one is processed
+  // (a single wave has nothing else to hide a load behind)
+  constexpr int TBATCH = 8;
+  float kn[TBATCH][NR], qn[TBATCH][NR], vn[TBATCH], ign[TBATCH], fgn[TBATCH];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int j = 0; j < TBATCH; ++j) {
+      const int t = min(t0 + j, b - 1);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        const int d = lane + 64 * i;
+        kn[j][i] = d < dk ? ldf(k + t * row_stride + h * dk + d) : 0.f;
+        qn[j][i] = d < dk ? ldf(q + t * row_stride + h * dk + d) * qscale : 0.f;
+      }
+      vn[j] = cok ? ldf(v + t * row_stride + h * dv + col) : 0.f;
+      ign[j] = gates[(int64_t)t * 2 * H + h];
+      fgn[j] = gates[(int64_t)t * 2 * H + H + h];
+    }
+  };
+  fetch(a);
+  for (int t0 = a; t0 < b; t0 += TBATCH) {
+    float kc[TBATCH][NR], qc[TBATCH][NR], vc[TBATCH], igc[TBATCH], fgc[TBATCH];
+#pragma unroll
+    for (int j = 0; j < TBATCH; ++j) {
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        kc[j][i] = kn[j][i];
+        qc[j][i] = qn[j][i];
+      }
+      vc[j] = vn[j];
+      igc[j] = ign[j];
+      fgc[j] = fgn[j];
+    }
+    if (t0 + TBATCH < b) fetch(t0 + TBATCH);
+#pragma unroll
+    for (int j = 0; j < TBATCH; ++j) {
+      const int t = t0 + j;
+      if (t < b) {
+        float* ks = kq[j & 1];
+        float* qs = ks + DP;
+        float nq = 0.f;
+        const float mn = fmaxf(fgc[j] + m, igc[j]);
+        const float da = __expf(fgc[j] + m - mn), db = __expf(igc[j] - mn);
+        m = mn;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          ks[lane + 64 * i] = kc[j][i];
+          qs[lane + 64 * i] = qc[j][i];
+          nr[i] = da * nr[i] + db * kc[j][i];
+          nq += nr[i] * qc[j][i];
+        }
+        __builtin_amdgcn_wave_barrier();
+        const float bv = db * vc[j];
+        float num[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 0; d < DK; d += 4) {
+          if (d < dk) {  // rows past dk hold zeros in k and q: a partly used group of four is harmless
+            const float4 k4 = *reinterpret_cast<const float4*>(ks + d);
+            const float4 q4 = *reinterpret_cast<const float4*>(qs + d);
+            S[d] = da * S[d] + k4.x * bv;
+            S[d + 1] = da * S[d + 1] + k4.y * bv;
+            S[d + 2] = da * S[d + 2] + k4.z * bv;
+            S[d + 3] = da * S[d + 3] + k4.w * bv;
+            num[0] += S[d] * q4.x;
+            num[1] += S[d + 1] * q4.y;
+            num[2] += S[d + 2] * q4.z;
+            num[3] += S[d + 3] * q4.w;
+          }
+        }
+        nq = wave_sum_dpp(nq);
+        if (cok)
+          out[((int64_t)t * H + h) * dv + col] = ((num[0] + num[1]) + (num[2] + num[3])) / (fmaxf(fabsf(nq), __expf(-mn)) + 1e-6f);
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < DK; ++d)
+    if (cok && d < dk) Sb[(int64_t)d * dv + col] = S[d];
+  if (blockIdx.z == 0) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+      if (lane + 64 * i < dk) nb[lane + 64 * i] = nr[i];
+    if (lane == 0) mp[slot * H + h] = m;
+  }
+}
+
 template <typename T, int DS>  // DS: rows per slab held in registers (>= ceil(dk / 4))
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                                                          int64_t row_stride, const float* __restrict__ gates,
-                                                         const float* __restrict__ b_i, const float* __restrict__ b_f, float cap,
                                                          float qscale, float* __restrict__ Sp, float* __restrict__ np,
                                                          float* __restrict__ mp, const int* __restrict__ slots,
                                                          const int* __restrict__ cu, const int* __restrict__ start,
@@ -45,7 +189,6 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ q
     nr[i] = (!fresh && r < rows && d0 + r < dk) ? nb[d0 + r] : 0.f;
   }
   float m = fresh ? 0.f : mp[slot * H + h];
-  const float bi = b_i[h], bf = b_f[h];
   for (int t = a; t < b; ++t) {
     const int buf = (t - a) & 1;
     float* qs = qk + buf * 2 * dk;
@@ -55,8 +198,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ q
       ks[d] = ldf(k + t * row_stride + h * dk + d);
     }
     const float vv = cok ? ldf(v + t * row_stride + h * dv + col) : 0.f;
-    const float ig = cap * tanhf((gates[(int64_t)t * 2 * H + h] + bi) / cap);
-    const float fg = log_sigmoid(cap * tanhf((gates[(int64_t)t * 2 * H + H + h] + bf) / cap));
+    const float ig = gates[(int64_t)t * 2 * H + h], fg = gates[(int64_t)t * 2 * H + H + h];
     const float mn = fmaxf(fg + m, ig);
     const float da = expf(fg + m - mn), db = expf(ig - mn);
     m = mn;
@@ -111,7 +253,7 @@ static void check_thd(const at::Tensor& t, int64_t T, int64_t H, int64_t d, int6
 
 at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
                       const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
-                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start) {
+                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab) {
   HYB_CHECK(q.is_cuda() && q.dim() == 3 && v.dim() == 3, "q, k [T, H, dk], v [T, H, dv]");
   const int64_t T = q.size(0), H = q.size(1), dk = q.size(2), dv = v.size(2);
   const int64_t rs = T > 1 ? q.stride(0) : 0;
@@ -131,6 +273,12 @@ at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
   c10::DeviceGuard guard(q.device());
   at::Tensor out = at::empty({T, H, dv}, q.options().dtype(at::kFloat));
   if (T == 0 || ns == 0) return out;
+  at::Tensor act = at::empty_like(gates);
+  {
+    const int64_t ng = T * 2 * H;
+    mlstm_gates_kernel<<<dim3((unsigned)((ng + 255) / 256)), 256, 0, cur_stream()>>>(gates.data_ptr<float>(), b_i.data_ptr<float>(),
+                                                                                    b_f.data_ptr<float>(), (float)cap, act.data_ptr<float>(), T, (int)H);
+  }
   const int rows = (int)((dk + 3) / 4);
   const size_t lds = (size_t)(4 * dk + 2 * 4 * 65) * sizeof(float);
   dim3 grid((unsigned)ns, (unsigned)H, (unsigned)((dv + 63) / 64));
@@ -138,13 +286,18 @@ at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
   HYB_CHECK(T <= 1 || (k.stride(0) == row_stride && v.stride(0) == row_stride), "q, k, v: the same row stride");
   dispatch_act(q, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    auto launch = [&](auto kern) {
-      kern<<<grid, 256, lds, cur_stream()>>>((const Tt*)q.data_ptr(), (const Tt*)k.data_ptr(), (const Tt*)v.data_ptr(), row_stride,
-                                            gates.data_ptr<float>(), b_i.data_ptr<float>(), b_f.data_ptr<float>(), (float)cap, (float)qscale,
-                                            S.data_ptr<float>(), n.data_ptr<float>(), m.data_ptr<float>(), slots.data_ptr<int>(),
-                                            cu.data_ptr<int>(), start.data_ptr<int>(), out.data_ptr<float>(), (int)H, (int)dk, (int)dv);
+    auto go = [&](auto kern, int threads, size_t shm) {
+      kern<<<grid, threads, shm, cur_stream()>>>((const Tt*)q.data_ptr(), (const Tt*)k.data_ptr(), (const Tt*)v.data_ptr(), row_stride,
+                                                act.data_ptr<float>(), (float)qscale, S.data_ptr<float>(), n.data_ptr<float>(),
+                                                m.data_ptr<float>(), slots.data_ptr<int>(), cu.data_ptr<int>(), start.data_ptr<int>(),
+                                                out.data_ptr<float>(), (int)H, (int)dk, (int)dv);
     };
-    if (rows <= 8) launch(mlstm_scan_kernel<Tt, 8>);
+    auto launch = [&](auto kern) { go(kern, 256, lds); };
+    if (!slab && dk <= 16) go(mlstm_scan_wave_kernel<Tt, 16>, 64, 0);
+    else if (!slab && dk <= 32) go(mlstm_scan_wave_kernel<Tt, 32>, 64, 0);
+    else if (!slab && dk <= 64) go(mlstm_scan_wave_kernel<Tt, 64>, 64, 0);
+    else if (!slab && dk <= 128) go(mlstm_scan_wave_kernel<Tt, 128>, 64, 0);
+    else if (rows <= 8) launch(mlstm_scan_kernel<Tt, 8>);
     else if (rows <= 16) launch(mlstm_scan_kernel<Tt, 16>);
     else if (rows <= 32) launch(mlstm_scan_kernel<Tt, 32>);
     else if (rows <= 64) launch(mlstm_scan_kernel<Tt, 64>);

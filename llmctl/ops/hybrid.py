@@ -92,11 +92,12 @@ def sigmoid_gate_mul(o, g):
     return ref.sigmoid_gate_mul(o, g)
 
 
-def mlstm_scan(q, k, v, if_raw, b_i, b_f, cap: float, qscale: float, S, n, m, state_slots, cu, start):
+def mlstm_scan(q, k, v, if_raw, b_i, b_f, cap: float, qscale: float, S, n, m, state_slots, cu, start, slab: bool = False):
     """mLSTM recurrence over the step's tokens; returns the un-normalised head outputs fp32
-    ``[T, H, dv]`` and updates the state pools in place."""
+    ``[T, H, dv]`` and updates the state pools in place.  ``slab`` forces the block-per-tile kernel
+    (the form for key dims above 128) where the wave-per-tile one would run."""
     if use_native(q):
-        return native_hybrid().mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu, start)
+        return native_hybrid().mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu, start, slab)
     return ref.mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu, start)
 
 

@@ -358,3 +358,52 @@ def test_checkpoint_names_round_trip(tmp_path):
     bad["l1.mix.uk"] = bad["l1.mix.uk"][:-1]
     with pytest.raises(ValueError):
         m.load_named(bad)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,dk,dv", [(3, 5, 7), (2, 20, 70), (1, 64, 64), (2, 100, 130), (1, 130, 40), (1, 300, 65)])
+def test_mlstm_scan_kernels_gpu(H, dk, dv):
+    # three sequences in one launch: a fresh one, a continued one and a single token; carried state;
+    # both kernel forms, against a direct float64 token loop
+    from llmctl.ops import hybrid
+
+    g = torch.Generator().manual_seed(dk)
+    T, cap, qs = 40, 6.0, dk ** -0.5
+    cu, start, slots = [0, 25, 39, 40], [0, 11, 3], [2, 0, 3]
+    z = torch.randn(T, 2 * H * dk + H * dv + 3, generator=g).bfloat16().float()
+    raw = torch.randn(T, 2 * H, generator=g) * 2
+    b_i, b_f = torch.randn(H, generator=g), torch.randn(H, generator=g) + 2
+    S0, n0, m0 = torch.randn(4, H, dk, dv, generator=g), torch.randn(4, H, dk, generator=g), torch.randn(4, H, generator=g)
+
+    def cut(t):
+        return (t[:, :H * dk].view(T, H, dk), t[:, H * dk:2 * H * dk].view(T, H, dk),
+                t[:, 2 * H * dk:2 * H * dk + H * dv].view(T, H, dv))
+
+    q, k, v = (x.double() for x in cut(z))
+    ig = cap * torch.tanh((raw.double()[:, :H] + b_i.double()) / cap)
+    fg = torch.nn.functional.logsigmoid(cap * torch.tanh((raw.double()[:, H:] + b_f.double()) / cap))
+    want = torch.zeros(T, H, dv, dtype=torch.float64)
+    Sw, nw, mw = S0.double().clone(), n0.double().clone(), m0.double().clone()
+    for s in range(3):
+        sl = slots[s]
+        S, n, m = ((torch.zeros_like(x[sl]) if start[s] == 0 else x[sl].clone()) for x in (Sw, nw, mw))
+        for t in range(cu[s], cu[s + 1]):
+            mn = torch.maximum(fg[t] + m, ig[t])
+            da, db = torch.exp(fg[t] + m - mn), torch.exp(ig[t] - mn)
+            S = da[:, None, None] * S + db[:, None, None] * k[t][:, :, None] * v[t][:, None, :]
+            n = da[:, None] * n + db[:, None] * k[t]
+            m = mn
+            den = torch.maximum((n * q[t] * qs).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            want[t] = torch.einsum("hkv,hk->hv", S, q[t] * qs) / den[:, None]
+        Sw[sl], nw[sl], mw[sl] = S, n, m
+    for dtype in (torch.float32, torch.bfloat16):
+        for slab in (False, True):
+            zd = z.to(dtype).cuda()
+            qd, kd, vd = cut(zd)
+            Sd, nd, md = S0.clone().cuda(), n0.clone().cuda(), m0.clone().cuda()
+            i32 = lambda a: torch.tensor(a, dtype=torch.int32).cuda()
+            got = hybrid.mlstm_scan(qd, kd, vd, raw.cuda(), b_i.cuda(), b_f.cuda(), cap, qs, Sd, nd, md, i32(slots), i32(cu),
+                                    i32(start), slab)
+            for name, a, b in (("out", got, want), ("S", Sd, Sw), ("n", nd, nw), ("m", md, mw)):
+                err = (a.double().cpu() - b).abs().max() / b.abs().max()
+                assert err < 2e-5, (dtype, slab, name, float(err))
