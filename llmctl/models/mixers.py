@@ -46,6 +46,7 @@ class StepBatch:
     start: torch.Tensor  # int32 [n]
     state: torch.Tensor  # int32 [n]
     max_q: int = 0  # the longest prompt portion of the step
+    cu_host: Optional[list] = None  # ``cu`` on the host (chunk-parallel scans split long portions)
 
 
 def _init(t: torch.Tensor, std: float) -> None:
@@ -136,5 +137,5 @@ class MLSTM(nn.Module):
         gates = F.linear(h.float(), self.w_if)  # fp32 [T, 2H]
         S, n, m = state
         o = hops.mlstm_scan(q, k, v, gates, self.b_i, self.b_f, self.cap, 1.0 / math.sqrt(dk), S, n, m, b.state,
-                            b.cu, b.start)
+                            b.cu, b.start, cu_host=b.cu_host)
         return F.linear(hops.headnorm_gate(o, self.norm, g, self.eps, h.dtype), self.w_o)

@@ -22,7 +22,11 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
                               int64_t window, const at::Tensor& sink, double scale, int64_t rk, bool mfma);
 at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
                       const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
-                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab);
+                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab,
+                      const c10::optional<at::Tensor>& fsum, bool write_out);
+void mlstm_chunk_combine(const at::Tensor& S, const at::Tensor& n, const at::Tensor& m, const at::Tensor& slots, const at::Tensor& start,
+                         const at::Tensor& base, const at::Tensor& locS, const at::Tensor& locn, const at::Tensor& locm,
+                         const at::Tensor& fsum, at::Tensor iS, at::Tensor in_, at::Tensor im);
 std::tuple<at::Tensor, at::Tensor> group_topk_router(const at::Tensor& logits, int64_t top, int64_t groups, int64_t keep);
 }  // namespace llmctl_hybrid
 
@@ -38,7 +42,8 @@ TORCH_LIBRARY(llmctl_hybrid, m) {
   m.def("latent_q_assemble(Tensor q_lat, Tensor q, Tensor pos, Tensor inv_freq, int rot_dims, int dn) -> Tensor");
   m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor sink, float scale, int rk, int max_q, bool mfma=True) -> Tensor");
   m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor sink, float scale, int rk, bool mfma=True) -> Tensor");
-  m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start, bool slab=False) -> Tensor");
+  m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start, bool slab=False, Tensor(d!)? fsum=None, bool write_out=True) -> Tensor");
+  m.def("mlstm_chunk_combine(Tensor S, Tensor n, Tensor m, Tensor slots, Tensor start, Tensor base, Tensor locS, Tensor locn, Tensor locm, Tensor fsum, Tensor(a!) iS, Tensor(b!) in_, Tensor(c!) im) -> ()");
   m.def("group_topk_router(Tensor logits, int top, int groups, int keep) -> (Tensor, Tensor)");
 }
 
@@ -55,5 +60,6 @@ TORCH_LIBRARY_IMPL(llmctl_hybrid, CUDA, m) {
   m.impl("latent_attn_prefill", &llmctl_hybrid::latent_attn_prefill);
   m.impl("latent_attn_decode", &llmctl_hybrid::latent_attn_decode);
   m.impl("mlstm_scan", &llmctl_hybrid::mlstm_scan);
+  m.impl("mlstm_chunk_combine", &llmctl_hybrid::mlstm_chunk_combine);
   m.impl("group_topk_router", &llmctl_hybrid::group_topk_router);
 }

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(64) void mlstm_scan_wave_kernel(const T* __restrict
                                                              float* __restrict__ Sp, float* __restrict__ np, float* __restrict__ mp,
                                                              const int* __restrict__ slots, const int* __restrict__ cu,
                                                              const int* __restrict__ start, float* __restrict__ out, int H, int dk,
-                                                             int dv) {
+                                                             int dv, float* __restrict__ fsum, int write_out) {
   constexpr int NR = (DK + 63) / 64;
   constexpr int DP = NR * 64;
   __shared__ __attribute__((aligned(16))) float kq[2][2 * DP];
@@ -63,13 +63,15 @@ __global__ __launch_bounds__(64) void mlstm_scan_wave_kernel(const T* __restrict
   const int64_t slot = slots[sq];
   float* Sb = Sp + (slot * H + h) * (int64_t)dk * dv;
   float* nb = np + (slot * H + h) * (int64_t)dk;
-  const bool fresh = start[sq] == 0;
+  const int st = start[sq];  // 0: new sequence (zero state, m = 0); -1: zero state with m = -inf (a chunk's
+  const bool fresh = st <= 0;  // own contribution, to be merged into the carried state); else: load the slot
   float S[DK], nr[NR];
 #pragma unroll
   for (int d = 0; d < DK; ++d) S[d] = (!fresh && cok && d < dk) ? Sb[(int64_t)d * dv + col] : 0.f;
 #pragma unroll
   for (int i = 0; i < NR; ++i) nr[i] = (!fresh && lane + 64 * i < dk) ? nb[lane + 64 * i] : 0.f;
-  float m = fresh ? 0.f : mp[slot * H + h];
+  float m = fresh ? (st < 0 ? -INFINITY : 0.f) : mp[slot * H + h];
+  float facc = 0.f;
   // operands of TBATCH tokens are loaded ahead, one batch in flight while the previous one is processed
   // (a single wave has nothing else to hide a load behind)
   constexpr int TBATCH = 8;
@@ -114,6 +116,7 @@ __global__ __launch_bounds__(64) void mlstm_scan_wave_kernel(const T* __restrict
         const float mn = fmaxf(fgc[j] + m, igc[j]);
         const float da = __expf(fgc[j] + m - mn), db = __expf(igc[j] - mn);
         m = mn;
+        facc += fgc[j];
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
           ks[lane + 64 * i] = kc[j][i];
@@ -140,7 +143,7 @@ __global__ __launch_bounds__(64) void mlstm_scan_wave_kernel(const T* __restrict
           }
         }
         nq = wave_sum_dpp(nq);
-        if (cok)
+        if (cok && write_out)
           out[((int64_t)t * H + h) * dv + col] = ((num[0] + num[1]) + (num[2] + num[3])) / (fmaxf(fabsf(nq), __expf(-mn)) + 1e-6f);
         __builtin_amdgcn_wave_barrier();
       }
@@ -153,7 +156,46 @@ __global__ __launch_bounds__(64) void mlstm_scan_wave_kernel(const T* __restrict
 #pragma unroll
     for (int i = 0; i < NR; ++i)
       if (lane + 64 * i < dk) nb[lane + 64 * i] = nr[i];
-    if (lane == 0) mp[slot * H + h] = m;
+    if (lane == 0) {
+      mp[slot * H + h] = m;
+      if (fsum != nullptr) fsum[(int64_t)sq * H + h] = facc;
+    }
+  }
+}
+
+// Merge per-chunk contributions into carried states.  Sequence s has chunks [base[s], base[s+1]); chunk
+// p's own contribution (run from a zero state with m = -inf) is (locS, locn, locm)[p] with summed log
+// forget gates fsum[p].  For every chunk the state at its first token is written to (iS, in, im)[p]:
+// the sequence's carried state for its first chunk, then m' = max(F + m, m_loc),
+// S' = e^(F + m - m') S + e^(m_loc - m') S_loc.  One thread per state entry, chunks in order.
+__global__ void mlstm_chunk_combine_kernel(const float* __restrict__ Sp, const float* __restrict__ np, const float* __restrict__ mp,
+                                           const int* __restrict__ slots, const int* __restrict__ start, const int* __restrict__ base,
+                                           const float* __restrict__ locS, const float* __restrict__ locn, const float* __restrict__ locm,
+                                           const float* __restrict__ fsum, float* __restrict__ iS, float* __restrict__ in_,
+                                           float* __restrict__ im, int H, int dk, int dv) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int64_t per = (int64_t)dk * dv + dk;  // S entries, then n entries
+  const int64_t e = (int64_t)blockIdx.z * blockDim.x + threadIdx.x;
+  if (e >= per) return;
+  const bool isn = e >= (int64_t)dk * dv;
+  const int64_t eo = isn ? e - (int64_t)dk * dv : e;
+  const int64_t stride = isn ? dk : (int64_t)dk * dv;
+  const float* real = isn ? np : Sp;
+  const float* loc = isn ? locn : locS;
+  float* init = isn ? in_ : iS;
+  const int64_t slot = slots[s];
+  const bool fresh = start[s] == 0;
+  float val = fresh ? 0.f : real[(slot * H + h) * stride + eo];
+  float m = fresh ? 0.f : mp[slot * H + h];
+  for (int p = base[s]; p < base[s + 1]; ++p) {
+    init[((int64_t)p * H + h) * stride + eo] = val;
+    if (e == 0) im[(int64_t)p * H + h] = m;
+    if (p + 1 < base[s + 1]) {
+      const float F = fsum[(int64_t)p * H + h], ml = locm[(int64_t)p * H + h];
+      const float mn = fmaxf(F + m, ml);
+      val = expf(F + m - mn) * val + expf(ml - mn) * loc[((int64_t)p * H + h) * stride + eo];
+      m = mn;
+    }
   }
 }
 
@@ -163,7 +205,8 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ q
                                                          float qscale, float* __restrict__ Sp, float* __restrict__ np,
                                                          float* __restrict__ mp, const int* __restrict__ slots,
                                                          const int* __restrict__ cu, const int* __restrict__ start,
-                                                         float* __restrict__ out, int H, int dk, int dv) {
+                                                         float* __restrict__ out, int H, int dk, int dv, float* __restrict__ fsum,
+                                                         int write_out) {
   extern __shared__ float sm[];
   float* qk = sm;                    // [2][2 dk]
   float* part = sm + 4 * dk;         // [2][4][65]
@@ -226,7 +269,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ q
     pp[lane] = num;
     if (lane == 0) pp[64] = nq;
     __syncthreads();
-    if (slab == 0 && cok) {
+    if (slab == 0 && cok && write_out) {
       const float* p0 = part + buf * 4 * 65;
       const float tot = p0[lane] + p0[65 + lane] + p0[130 + lane] + p0[195 + lane];
       const float nqt = p0[64] + p0[65 + 64] + p0[130 + 64] + p0[195 + 64];
@@ -253,7 +296,8 @@ static void check_thd(const at::Tensor& t, int64_t T, int64_t H, int64_t d, int6
 
 at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
                       const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
-                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab) {
+                      const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab,
+                      const c10::optional<at::Tensor>& fsum, bool write_out) {
   HYB_CHECK(q.is_cuda() && q.dim() == 3 && v.dim() == 3, "q, k [T, H, dk], v [T, H, dv]");
   const int64_t T = q.size(0), H = q.size(1), dk = q.size(2), dv = v.size(2);
   const int64_t rs = T > 1 ? q.stride(0) : 0;
@@ -270,6 +314,10 @@ at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
   for (const at::Tensor* t : {&slots, &cu, &start}) HYB_CHECK(t->is_cuda() && t->is_contiguous() && t->scalar_type() == at::kInt, "slots / cu / start: int32");
   HYB_CHECK(cu.numel() == ns + 1 && start.numel() == ns, "cu [n + 1], start [n], slots [n]");
   HYB_CHECK(dk >= 1 && dk <= 512 && H <= 65535, "dk <= 512");
+  const bool wave = !slab && dk <= 128;
+  if (fsum.has_value())
+    HYB_CHECK(wave && fsum->is_cuda() && fsum->is_contiguous() && fsum->scalar_type() == at::kFloat && fsum->numel() == ns * H,
+              "fsum: fp32 [n, H], wave-per-tile form only (dk <= 128)");
   c10::DeviceGuard guard(q.device());
   at::Tensor out = at::empty({T, H, dv}, q.options().dtype(at::kFloat));
   if (T == 0 || ns == 0) return out;
@@ -290,7 +338,8 @@ at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
       kern<<<grid, threads, shm, cur_stream()>>>((const Tt*)q.data_ptr(), (const Tt*)k.data_ptr(), (const Tt*)v.data_ptr(), row_stride,
                                                 act.data_ptr<float>(), (float)qscale, S.data_ptr<float>(), n.data_ptr<float>(),
                                                 m.data_ptr<float>(), slots.data_ptr<int>(), cu.data_ptr<int>(), start.data_ptr<int>(),
-                                                out.data_ptr<float>(), (int)H, (int)dk, (int)dv);
+                                                out.data_ptr<float>(), (int)H, (int)dk, (int)dv,
+                                                fsum.has_value() ? fsum->data_ptr<float>() : nullptr, write_out ? 1 : 0);
     };
     auto launch = [&](auto kern) { go(kern, 256, lds); };
     if (!slab && dk <= 16) go(mlstm_scan_wave_kernel<Tt, 16>, 64, 0);
@@ -304,6 +353,25 @@ at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
     else launch(mlstm_scan_kernel<Tt, 128>);
   });
   return out;
+}
+
+void mlstm_chunk_combine(const at::Tensor& S, const at::Tensor& n, const at::Tensor& m, const at::Tensor& slots, const at::Tensor& start,
+                         const at::Tensor& base, const at::Tensor& locS, const at::Tensor& locn, const at::Tensor& locm,
+                         const at::Tensor& fsum, at::Tensor iS, at::Tensor in_, at::Tensor im) {
+  HYB_CHECK(S.is_cuda() && S.dim() == 4 && locS.dim() == 4 && iS.sizes() == locS.sizes() && in_.sizes() == locn.sizes() && im.sizes() == locm.sizes(), "state pools");
+  const int64_t H = S.size(1), dk = S.size(2), dv = S.size(3), P = locS.size(0), ns = slots.numel();
+  HYB_CHECK(locS.size(1) == H && locS.size(2) == dk && locS.size(3) == dv && locn.size(0) == P && locm.size(0) == P && fsum.numel() == P * H, "chunk pools [P, H, ...]");
+  for (const at::Tensor* t : std::initializer_list<const at::Tensor*>{&S, &n, &m, &locS, &locn, &locm, &fsum, &iS, &in_, &im})
+    HYB_CHECK(t->is_cuda() && t->is_contiguous() && t->scalar_type() == at::kFloat, "contiguous fp32 GPU tensors");
+  for (const at::Tensor* t : {&slots, &start, &base}) HYB_CHECK(t->is_cuda() && t->is_contiguous() && t->scalar_type() == at::kInt, "int32 metadata");
+  HYB_CHECK(start.numel() == ns && base.numel() == ns + 1, "start [n], base [n + 1]");
+  if (ns == 0 || P == 0) return;
+  c10::DeviceGuard guard(S.device());
+  const int64_t per = dk * dv + dk;
+  dim3 grid((unsigned)ns, (unsigned)H, (unsigned)((per + 255) / 256));
+  mlstm_chunk_combine_kernel<<<grid, 256, 0, cur_stream()>>>(S.data_ptr<float>(), n.data_ptr<float>(), m.data_ptr<float>(), slots.data_ptr<int>(),
+      start.data_ptr<int>(), base.data_ptr<int>(), locS.data_ptr<float>(), locn.data_ptr<float>(), locm.data_ptr<float>(), fsum.data_ptr<float>(),
+      iS.data_ptr<float>(), in_.data_ptr<float>(), im.data_ptr<float>(), (int)H, (int)dk, (int)dv);
 }
 
 }  // namespace llmctl_hybrid

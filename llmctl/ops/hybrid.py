@@ -92,13 +92,62 @@ def sigmoid_gate_mul(o, g):
     return ref.sigmoid_gate_mul(o, g)
 
 
-def mlstm_scan(q, k, v, if_raw, b_i, b_f, cap: float, qscale: float, S, n, m, state_slots, cu, start, slab: bool = False):
+MLSTM_CHUNK = 128  # tokens per chunk of the chunk-parallel scan; portions of >= 2 chunks take it
+
+
+def mlstm_scan(q, k, v, if_raw, b_i, b_f, cap: float, qscale: float, S, n, m, state_slots, cu, start, slab: bool = False,
+               cu_host=None):
     """mLSTM recurrence over the step's tokens; returns the un-normalised head outputs fp32
     ``[T, H, dv]`` and updates the state pools in place.  ``slab`` forces the block-per-tile kernel
-    (the form for key dims above 128) where the wave-per-tile one would run."""
+    (the form for key dims above 128) where the wave-per-tile one would run.  ``cu_host`` (the row
+    offsets as a host list) lets long portions run chunk-parallel (:func:`_mlstm_scan_chunked`)."""
     if use_native(q):
+        if (cu_host is not None and not slab and q.shape[-1] <= 128
+                and max((b - a for a, b in zip(cu_host[:-1], cu_host[1:])), default=0) >= 2 * MLSTM_CHUNK):
+            return _mlstm_scan_chunked(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, start, cu_host)
         return native_hybrid().mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu, start, slab)
     return ref.mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, cu, start)
+
+
+def _mlstm_scan_chunked(q, k, v, if_raw, b_i, b_f, cap, qscale, S, n, m, state_slots, start, cu_host):
+    """The same token-by-token recurrence with the chunks of a portion running side by side.  The state
+    is linear in its past: over a chunk with summed log forget gates F and own contribution (S_loc, m_loc)
+    -- the chunk run from a zero state with m = -inf -- the carried state becomes m' = max(F + m, m_loc),
+    S' = e^(F + m - m') S + e^(m_loc - m') S_loc, and m' is exactly the stabiliser the sequential run
+    reaches.  Three passes: (1) every chunk's own contribution, all chunks at once, no outputs; (2) the
+    states at every chunk's first token, chunk after chunk (elementwise); (3) every chunk again from its
+    true state, all at once, writing the outputs token by token as the sequential form does.  A single
+    prompt thus fills chunks x heads x value-tiles waves instead of heads x value-tiles."""
+    nat = native_hybrid()
+    dev = q.device
+    H, dk, dv = q.shape[1], q.shape[2], v.shape[2]
+    pcu, base = [0], [0]
+    for a, b in zip(cu_host[:-1], cu_host[1:]):
+        t = a
+        while t < b:
+            t = min(t + MLSTM_CHUNK, b)
+            pcu.append(t)
+        base.append(len(pcu) - 1)
+    P = len(pcu) - 1
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32).to(dev, non_blocking=True)
+    pcu_d, base_d, ident = i32(pcu), i32(base), torch.arange(P, dtype=torch.int32, device=dev)
+    f32 = dict(dtype=torch.float32, device=dev)
+    locS, locn, locm = torch.empty(P, H, dk, dv, **f32), torch.empty(P, H, dk, **f32), torch.empty(P, H, **f32)
+    fsum = torch.empty(P, H, **f32)
+    nat.mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, locS, locn, locm, ident, pcu_d,
+                   torch.full((P,), -1, dtype=torch.int32, device=dev), False, fsum, False)
+    iS, in_, im = torch.empty_like(locS), torch.empty_like(locn), torch.empty_like(locm)
+    nat.mlstm_chunk_combine(S, n, m, state_slots, start, base_d, locS, locn, locm, fsum, iS, in_, im)
+    out = nat.mlstm_scan(q, k, v, if_raw, b_i, b_f, cap, qscale, iS, in_, im, ident, pcu_d,
+                         torch.ones(P, dtype=torch.int32, device=dev), False, None, True)
+    live = [s for s in range(len(base) - 1) if base[s + 1] > base[s]]
+    if live:  # the last chunk's final state is the sequence's new carried state
+        last = torch.tensor([base[s + 1] - 1 for s in live], dtype=torch.long).to(dev, non_blocking=True)
+        dst = state_slots.long()[torch.tensor(live, dtype=torch.long).to(dev, non_blocking=True)]
+        S.index_copy_(0, dst, iS.index_select(0, last))
+        n.index_copy_(0, dst, in_.index_select(0, last))
+        m.index_copy_(0, dst, im.index_select(0, last))
+    return out
 
 
 def headnorm_gate(o, w, g, eps: float, out_dtype):

@@ -222,7 +222,7 @@ class InferenceEngine:
                           p_cu=i32(p_cu) if Tp else None, p_ctx=i32(pp["ctx"]) if Tp else None,
                           p_bt=i32(pp["bt"]) if Tp else None, d_ctx=i32(dp["ctx"]) if Td else None,
                           d_bt=i32(dp["bt"]) if Td else None, cu=i32(cu), start=i32(start), state=i32(state),
-                          max_q=max((b - a for a, b in zip(p_cu[:-1], p_cu[1:])), default=0))
+                          max_q=max((b - a for a, b in zip(p_cu[:-1], p_cu[1:])), default=0), cu_host=cu)
         if rows is None:
             rows = (list(pp["last"]) if Tp else []) + list(range(Tp, Tp + Td))
         if count:

@@ -407,3 +407,14 @@ def test_mlstm_scan_kernels_gpu(H, dk, dv):
             for name, a, b in (("out", got, want), ("S", Sd, Sw), ("n", nd, nw), ("m", md, mw)):
                 err = (a.double().cpu() - b).abs().max() / b.abs().max()
                 assert err < 2e-5, (dtype, slab, name, float(err))
+
+
+def test_long_portions_in_one_step(tmp_path, dev):
+    # portions long enough for the chunk-parallel scan (several chunks, the last one partial) beside a
+    # short one and a decoded token; then decoding goes on from the carried state (no routed experts:
+    # among a thousand positions a near-tie of two experts would flip under bf16 rounding)
+    cfg = U.config([(U.rec(heads=2, dim=6, vdim=8), None), (U.attn(window=40), None)])
+    W = U.random_weights(cfg, 80, forget_bias=5.0)
+    r = {"a": tokens(700, 50, 81), "b": tokens(300, 50, 82), "c": tokens(9, 50, 83)}
+    steps = [[("c", 8)], [("a", 300), ("b", 290), ("c", 1)], [("a", 397), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 3 + [[("b", 6)]]
+    check(tmp_path, dev, cfg, r, steps, W=W, blocks=80, block_size=16)
