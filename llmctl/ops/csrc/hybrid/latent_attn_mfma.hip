@@ -94,20 +94,31 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   constexpr int CPT = NCB * 16;  // 16-byte chunks of one key row (padded R)
   for (int t = t_lo; t < t_hi; ++t) {
     __syncthreads();
+    // four 16-byte pieces in flight per lane at a time: the whole row set at once would cost 4 NCB
+    // registers x 4 on top of the Q fragments and the accumulators
+#pragma unroll 1
+    for (int it0 = 0; it0 < NCB * 4; it0 += 4) {
+      uint4 v[4];
 #pragma unroll
-    for (int it = 0; it < NCB * 4; ++it) {
-      const int c = tid + 256 * it;
-      const int krow = c / CPT, ch = c % CPT;
-      const int key = t * LKB + krow, col = ch * 8;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (key < ctx && col < a.R) {
-        const long slot = (long)btn[key / a.bs] * a.bs + key % a.bs;
-        v = gload16(a.cache + slot * a.R + col);
+      for (int j = 0; j < 4; ++j) {
+        const int c = tid + 256 * (it0 + j);
+        const int krow = c / CPT, ch = c % CPT;
+        const int key = t * LKB + krow, col = ch * 8;
+        v[j] = make_uint4(0, 0, 0, 0);
+        if (key < ctx && col < a.R) {
+          const long slot = (long)btn[key / a.bs] * a.bs + key % a.bs;
+          v[j] = gload16(a.cache + slot * a.R + col);
+        }
       }
-      const int cb = ch >> 4, chb = ch & 15;
-      *reinterpret_cast<uint4*>(Ks + cb * LIMG + row_off<128>(krow, chb)) = v;
-      const int tb = cb - v0 / 128;
-      if (tb >= 0 && tb < NTB) *reinterpret_cast<uint4*>(Vs + tb * LIMG + tr_off<128>(krow, chb)) = v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = tid + 256 * (it0 + j);
+        const int krow = c / CPT, ch = c % CPT;
+        const int cb = ch >> 4, chb = ch & 15;
+        *reinterpret_cast<uint4*>(Ks + cb * LIMG + row_off<128>(krow, chb)) = v[j];
+        const int tb = cb - v0 / 128;
+        if (tb >= 0 && tb < NTB) *reinterpret_cast<uint4*>(Vs + tb * LIMG + tr_off<128>(krow, chb)) = v[j];
+      }
     }
     __syncthreads();
     const int kv0 = t * LKB;
