@@ -37,6 +37,11 @@ struct LArgs {
   const float* sink;
   int H, R, rk, bs, maxb, window, HB, nvt;
   float scale_log2;
+  // decode rows with the key range split over blockIdx.x (few sequences would otherwise leave the chip
+  // idle): each split writes its unnormalised fp32 output and (running maximum, denominator) here
+  int nsplit;
+  float* ws_o;   // [rows, nsplit, rk]
+  float* ws_ml;  // [rows, nsplit, 2]
 };
 
 template <int NCB, int NDB>
@@ -55,7 +60,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int q_begin = a.cu ? a.cu[n] : n;
   const int qlen = a.cu ? a.cu[n + 1] - q_begin : 1;
   const int HB = a.HB, TB = 128 / HB;
-  const int tok0 = blockIdx.x * TB;
+  const int split = a.nsplit > 1 ? blockIdx.x : 0;
+  const int tok0 = a.nsplit > 1 ? 0 : blockIdx.x * TB;
   if (tok0 >= qlen) return;
   const int ctx = a.ctx[n];
   const int pos0 = ctx - qlen;
@@ -83,9 +89,18 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
   float m_i = a.sink[headc] * kLog2e, l_i = 1.0f;  // the sink: one unit of mass at its own logit
+  if (split > 0) {                                 // (counted by the first split only)
+    m_i = -INFINITY;
+    l_i = 0.f;
+  }
 
   const int first_pos = pos0 + tok0, last_pos = pos0 + min(tok0 + TB, qlen) - 1;
-  const int t_lo = max(0, first_pos - a.window + 1) / LKB, t_hi = last_pos / LKB + 1;
+  int t_lo = max(0, first_pos - a.window + 1) / LKB, t_hi = last_pos / LKB + 1;
+  if (a.nsplit > 1) {
+    const int per = (t_hi - t_lo + a.nsplit - 1) / a.nsplit;
+    t_lo += split * per;
+    t_hi = min(t_hi, t_lo + per);
+  }
   // this wave's rows: positions [w_first, w_last]
   const int w_first = pos0 + min(tok0 + (wave * 32) / HB, qlen - 1);
   const int w_last = pos0 + min(tok0 + (wave * 32 + 31) / HB, qlen - 1);
@@ -148,7 +163,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const bool grow = __builtin_amdgcn_ballot_w64(mx > m_i + kRescaleTh) != 0;
-    const float m_new = grow ? fmaxf(m_i, mx) : m_i;
+    const float m_raw = grow ? fmaxf(m_i, mx) : m_i;
+    const float m_new = m_raw == -INFINITY ? 0.f : m_raw;  // nothing seen yet (a later split, all keys masked)
     float rs = 0.f;
     bf16x8_t pb[2][2];
 #pragma unroll
@@ -172,7 +188,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
         for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
     }
     l_i += rs;
-    m_i = m_new;
+    m_i = m_raw;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -184,7 +200,21 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
         }
   }
 
-  if (valid) {
+  if (valid && a.nsplit > 1) {
+    const long rowi = (long)(q_begin + my_tok) * a.H + my_head;
+    float* Wp = a.ws_o + (rowi * a.nsplit + split) * a.rk;
+#pragma unroll
+    for (int d = 0; d < NDB; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int col = v0 + d * 32 + 8 * g + 4 * hh;
+        if (col < a.rk) *reinterpret_cast<float4*>(Wp + col) = make_float4(o[d][4 * g], o[d][4 * g + 1], o[d][4 * g + 2], o[d][4 * g + 3]);
+      }
+    if (v0 == 0 && hh == 0) {
+      a.ws_ml[(rowi * a.nsplit + split) * 2] = m_i;
+      a.ws_ml[(rowi * a.nsplit + split) * 2 + 1] = l_i;
+    }
+  } else if (valid) {
     const float inv = 1.f / l_i;
     unsigned short* Op = a.out + ((long)(q_begin + my_tok) * a.H + my_head) * a.rk;
 #pragma unroll
@@ -200,6 +230,24 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
               make_uint2((unsigned)w4[0] | ((unsigned)w4[1] << 16), (unsigned)w4[2] | ((unsigned)w4[3] << 16));
         }
       }
+  }
+}
+
+// out[row] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s (splits that saw nothing: m = -inf, l = 0)
+__global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, unsigned short* __restrict__ out,
+                                          int nsplit, int rk) {
+  const long row = blockIdx.x;
+  const float* ml = ws_ml + row * nsplit * 2;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[2 * s]);
+  float L = 0.f;
+  for (int s = 0; s < nsplit; ++s) L += ml[2 * s + 1] * (ml[2 * s] == -INFINITY ? 0.f : fast_exp2(ml[2 * s] - M));
+  const float inv = 1.f / L;
+  for (int c = threadIdx.x; c < rk; c += blockDim.x) {
+    float v = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+      if (ml[2 * s] != -INFINITY) v += ws_o[(row * nsplit + s) * rk + c] * fast_exp2(ml[2 * s] - M);
+    out[row * rk + c] = __bfloat16_as_ushort(__float2bfloat16(v * inv));
   }
 }
 
@@ -235,11 +283,24 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
   const int TB = 128 / HB;
   const int hgroups = (int)((H + HB - 1) / HB);
   HYB_CHECK(ns <= 65535 && hgroups * nvt <= 65535, "grid too large");
+  // decode rows: split the window's key tiles over workgroups until the launch has a few hundred of them
+  int nsplit = 1;
+  at::Tensor ws_o, ws_ml;
+  if (cu == nullptr && rk % 4 == 0) {
+    const int tiles = (int)((window + LKB - 1) / LKB) + 1;
+    const long blocks = (long)ns * hgroups * nvt;
+    while (nsplit < tiles && nsplit < 32 && blocks * nsplit < 512) nsplit *= 2;
+    if (nsplit > 1) {
+      ws_o = at::empty({ns * H, nsplit, rk}, qa.options().dtype(at::kFloat));
+      ws_ml = at::empty({ns * H, nsplit, 2}, qa.options().dtype(at::kFloat));
+    }
+  }
   LArgs a{reinterpret_cast<const unsigned short*>(qa.data_ptr()), reinterpret_cast<const unsigned short*>(cache.data_ptr()),
           reinterpret_cast<unsigned short*>(out.data_ptr()), bt.data_ptr<int>(), cu ? cu->data_ptr<int>() : nullptr, ctx.data_ptr<int>(),
           sink.data_ptr<float>(), (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
-          (float)(scale * 1.4426950408889634)};
-  dim3 grid((unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
+          (float)(scale * 1.4426950408889634), nsplit, nsplit > 1 ? ws_o.data_ptr<float>() : nullptr,
+          nsplit > 1 ? ws_ml.data_ptr<float>() : nullptr};
+  dim3 grid(nsplit > 1 ? (unsigned)nsplit : (unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
   hipStream_t st = cur_stream();
   switch (ncb) {
     case 1: launch_ncb<1>(a, ndb, grid, st); break;
@@ -248,6 +309,9 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
     case 4: launch_ncb<4>(a, ndb, grid, st); break;
     default: launch_ncb<5>(a, ndb, grid, st); break;
   }
+  if (nsplit > 1)
+    latent_split_merge_kernel<<<dim3((unsigned)(ns * H)), 128, 0, st>>>(ws_o.data_ptr<float>(), ws_ml.data_ptr<float>(),
+                                                                        reinterpret_cast<unsigned short*>(out.data_ptr()), nsplit, (int)rk);
 }
 
 }  // namespace llmctl_hybrid
