@@ -42,7 +42,7 @@ def start(
     p = Path(artifact)
     from llmctl.models.config import ALIASES
 
-    if not p.exists() and artifact.lower() not in ALIASES:
+    if not p.exists() and artifact.lower() not in ALIASES and not artifact.lower().startswith("lenitar-"):
         console.print(f"[red]Artifact not found: {artifact}[/red]")
         raise typer.Exit(1)
     console.print("[blue]Starting inference server...[/blue]")
@@ -74,6 +74,22 @@ def start(
         server.run()
     except KeyboardInterrupt:
         console.print("\n[yellow]Server stopped[/yellow]")
+
+
+@app.command()
+def trace(
+    model: str = typer.Option(..., help="Checkpoint directory (config.json + model.safetensors)"),
+    out: str = typer.Option(..., help="Directory for the <step>.f32 logit files"),
+    dtype: str = typer.Option("bfloat16", help="bfloat16 or float32"),
+    max_tokens: int = typer.Option(4096, help="Tokens the cache pool holds"),
+    max_seqs: int = typer.Option(4, help="Live sequences (state slots)"),
+    device: str = typer.Option("auto", help="Device (auto, cuda, cpu)"),
+) -> None:
+    """Replay a token trace (JSON steps on standard input) through the engine; writes the logits asked for."""
+    from llmctl.serve.trace_replay import main as replay
+
+    raise typer.Exit(replay(["--model", model, "--out", out, "--dtype", dtype, "--max-tokens", str(max_tokens),
+                             "--max-seqs", str(max_seqs), "--device", device]))
 
 
 @app.callback(invoke_without_command=True)
