@@ -106,35 +106,42 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int w_last = pos0 + min(tok0 + (wave * 32 + 31) / HB, qlen - 1);
   const bool wave_live = tok0 + (wave * 32) / HB < qlen && hg * HB + (HB >= 32 ? (wave * 32) % HB : 0) < a.H;
 
-  constexpr int CPT = NCB * 16;  // 16-byte chunks of one key row (padded R)
-  for (int t = t_lo; t < t_hi; ++t) {
-    __syncthreads();
-    // four 16-byte pieces in flight per lane at a time: the whole row set at once would cost 4 NCB
-    // registers x 4 on top of the Q fragments and the accumulators
-#pragma unroll 1
-    for (int it0 = 0; it0 < NCB * 4; it0 += 4) {
-      uint4 v[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int c = tid + 256 * (it0 + j);
-        const int krow = c / CPT, ch = c % CPT;
-        const int key = t * LKB + krow, col = ch * 8;
-        v[j] = make_uint4(0, 0, 0, 0);
-        if (key < ctx && col < a.R) {
-          const long slot = (long)btn[key / a.bs] * a.bs + key % a.bs;
-          v[j] = gload16(a.cache + slot * a.R + col);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int c = tid + 256 * (it0 + j);
-        const int krow = c / CPT, ch = c % CPT;
-        const int cb = ch >> 4, chb = ch & 15;
-        *reinterpret_cast<uint4*>(Ks + cb * LIMG + row_off<128>(krow, chb)) = v[j];
-        const int tb = cb - v0 / 128;
-        if (tb >= 0 && tb < NTB) *reinterpret_cast<uint4*>(Vs + tb * LIMG + tr_off<128>(krow, chb)) = v[j];
-      }
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned lds_base = lds_addr(smem);
+  // cache slots of a tile's 64 keys, looked up in the block table one tile ahead (double-buffered)
+  int* slot_lds = reinterpret_cast<int*>(smem + (NCB + NTB) * LIMG);
+  auto load_slots = [&](int t, int buf) {
+    if (tid < LKB) {
+      const int key = min(t * LKB + tid, ctx - 1);
+      slot_lds[buf * LKB + tid] = btn[key / a.bs] * a.bs + key % a.bs;
     }
+  };
+  if (t_lo < t_hi) load_slots(t_lo, 0);
+  for (int t = t_lo; t < t_hi; ++t) {
+    const int sbuf = (t - t_lo) & 1;
+    __syncthreads();
+    // LDS-DMA fill: every wave instruction moves 4 key rows x 256 B of one image straight from the cache
+    // to LDS (no registers, all pieces of the tile in flight at once); the images' swizzles are applied
+    // to the source chunk.  Keys past the context and columns past R read a valid neighbour instead
+    // (finite data): such keys are masked below and such columns meet zero Q entries or are never stored.
+#pragma unroll 4
+    for (int g = wave_u; g < 16 * (NCB + NTB); g += 4) {
+      const int img = g >> 4, rg = g & 15;
+      const int krow = rg * 4 + (lane >> 4), chp = lane & 15;
+      const long slot = slot_lds[sbuf * LKB + krow];
+      int cb, c;
+      if (img < NCB) {
+        cb = img;
+        c = chp ^ swz_row<128>(krow);
+      } else {
+        cb = v0 / 128 + (img - NCB);
+        c = chp ^ swz_tr<128>(krow);
+      }
+      const int col = min((cb * 16 + c) * 8, a.R - 8);
+      dma16(a.cache + slot * a.R + col, lds_base + (unsigned)(img * LIMG + rg * 1024));
+    }
+    if (t + 1 < t_hi) load_slots(t + 1, sbuf ^ 1);
+    vm_wait<0>();
     __syncthreads();
     const int kv0 = t * LKB;
     if (!wave_live || kv0 > w_last || kv0 + LKB - 1 < w_first - a.window + 1) continue;
@@ -254,7 +261,7 @@ __global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const 
 template <int NCB>
 void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
   auto go = [&](auto kern, int NDBv) {
-    const size_t lds = (size_t)(NCB + (NDBv + 3) / 4) * LIMG;
+    const size_t lds = (size_t)(NCB + (NDBv + 3) / 4) * LIMG + 2 * LKB * sizeof(int);
     HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
     kern<<<grid, 256, lds, st>>>(a);
   };
