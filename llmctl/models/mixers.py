@@ -6,6 +6,13 @@
   latent space once and attends the cache rows directly (one "head" of width ``rank + rot`` serves all
   query heads), and the value up-projection is applied to the attended latent afterwards.  Options:
   sliding window, a per-head softmax sink, a sigmoid output gate, a low-rank query path.
+* :class:`GroupedAttention` — grouped-query softmax attention over a paged row cache ``[v | k]`` per
+  kv head, with the options of small recent designs as parameters: short causal convolutions on the
+  projected q / k / v, per-head RMS norm of q and k, rotary positions (neighbour or half pairs, YaRN
+  frequency scaling), values turned by their position and the head outputs turned back, a learned
+  per-head temperature, chunked or windowed masks, a softmax sink.
+* :class:`CausalConv` — a short causal convolution over time per channel, its last inputs carried in a
+  state slot; :class:`ClampedGLU` — a gated feed-forward with clamped branches.
 * :class:`MLSTM` — the xLSTM matrix memory: per head a ``[dk, dv]`` state with exponential input gate,
   sigmoid forget gate (both soft-capped) and a running log-scale stabiliser; state lives in a slot
   pool of the engine's cache, one slot per live sequence.
@@ -47,6 +54,28 @@ class StepBatch:
     state: torch.Tensor  # int32 [n]
     max_q: int = 0  # the longest prompt portion of the step
     cu_host: Optional[list] = None  # ``cu`` on the host (chunk-parallel scans split long portions)
+    seq_of: Optional[torch.Tensor] = None  # int32 [T] index (into cu / start / state) of every row's sequence
+    d_max_ctx: int = 0  # the longest context among the decoding sequences
+
+
+def rotary_frequencies(base: float, dims: int, scaling: Optional[dict] = None, device=None):
+    """Per-pair rotary frequencies ``base^(-2i/dims)`` (fp32 ``[dims/2]``) and the factor on cos and sin.
+    ``scaling`` = ``{factor, original, fast, slow}`` applies YaRN: with ``where(t) = dims ln(original /
+    (2 pi t)) / (2 ln base)`` the pairs below ``floor(where(fast))`` keep their frequency, those above
+    ``ceil(where(slow))`` are divided by ``factor``, a linear ramp lies between; cos and sin are multiplied
+    by ``0.1 ln(factor) + 1``."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    amp = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        where = lambda t: dims * math.log(orig / (2.0 * math.pi * t)) / (2.0 * math.log(float(base)))
+        lo = max(math.floor(where(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(where(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        amp = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32).to(device), amp
 
 
 def _init(t: torch.Tensor, std: float) -> None:
@@ -55,29 +84,37 @@ def _init(t: torch.Tensor, std: float) -> None:
 
 
 class LatentAttention(nn.Module):
-    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, q_rank: int,
-                 rot_base: float, rot_dims: int, scale: float, window: int, eps: float, device=None, dtype=None):
+    """Options: ``q_rank`` None = a full-rank query projection; ``window`` None = plain causal; ``sink``
+    / ``gate`` False = no softmax sink / no sigmoid output gate; ``rot_scaling`` = YaRN (see
+    :func:`rotary_frequencies`); ``interleaved`` = rotary pairs are neighbours (2i, 2i+1), not halves."""
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, q_rank: Optional[int],
+                 rot_base: float, rot_dims: int, scale: float, window: Optional[int], eps: float, device=None, dtype=None,
+                 sink: bool = True, gate: bool = True, rot_scaling: Optional[dict] = None, interleaved: bool = False):
         super().__init__()
         self.width, self.H, self.dn, self.dr, self.dv = width, heads, dim, rot_dim, vdim
-        self.rk, self.qr, self.rot_dims, self.scale, self.window, self.eps = kv_rank, q_rank, rot_dims, scale, window, eps
+        self.rk, self.qr, self.rot_dims, self.scale, self.eps = kv_rank, q_rank, rot_dims, scale, eps
+        self.window = int(window) if window else hops.NO_LIMIT
+        self.has_gate, self.interleaved = gate, interleaved
         if rot_dims > rot_dim or rot_dims % 2:
             raise ValueError("rotary dims must be even and fit the rotated part")
         kw = dict(device=device, dtype=dtype)
         f32 = dict(device=device, dtype=torch.float32)
-        # one GEMM for everything that reads the layer input: [W_dq ; W_dkv ; W_g]
-        self.w_in = nn.Parameter(torch.empty(q_rank + kv_rank + rot_dim + heads * vdim, width, **kw))
-        self.w_uq = nn.Parameter(torch.empty(heads * (dim + rot_dim), q_rank, **kw))
+        # one GEMM for everything that reads the layer input: [W_dq or W_q ; W_dkv ; W_g]
+        self.q_cols = q_rank if q_rank else heads * (dim + rot_dim)
+        self.w_in = nn.Parameter(torch.empty(self.q_cols + kv_rank + rot_dim + (heads * vdim if gate else 0), width, **kw))
+        self.w_uq = nn.Parameter(torch.empty(heads * (dim + rot_dim), q_rank, **kw)) if q_rank else None
         self.w_uk = nn.Parameter(torch.empty(heads, dim, kv_rank, **kw))  # per head [dn, rank]
         self.w_uv = nn.Parameter(torch.empty(heads, vdim, kv_rank, **kw))  # per head [dv, rank]
         self.w_o = nn.Parameter(torch.empty(width, heads * vdim, **kw))
-        self.q_norm = nn.Parameter(torch.ones(q_rank, **f32))
+        self.q_norm = nn.Parameter(torch.ones(q_rank, **f32)) if q_rank else None
         self.kv_norm = nn.Parameter(torch.ones(kv_rank, **f32))
-        self.sink = nn.Parameter(torch.zeros(heads, **f32))
+        self.sink = nn.Parameter(torch.zeros(heads, **f32)) if sink else None
         for w in (self.w_in, self.w_uq, self.w_uk, self.w_uv, self.w_o):
-            _init(w, 0.02)
-        i = torch.arange(rot_dims // 2, dtype=torch.float64)
-        self.register_buffer("inv_freq", (float(rot_base) ** (-2.0 * i / rot_dims)).to(torch.float32).to(device),
-                             persistent=False)
+            if w is not None:
+                _init(w, 0.02)
+        inv_freq, self.rot_amp = rotary_frequencies(rot_base, rot_dims, rot_scaling, device)
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
 
     cache_kind = "latent"
 
@@ -85,25 +122,139 @@ class LatentAttention(nn.Module):
     def cache_row(self) -> int:
         return self.rk + self.dr
 
-    def step(self, h: torch.Tensor, b: StepBatch, cache: torch.Tensor) -> torch.Tensor:
+    def state_shapes(self):
+        return []
+
+    def step(self, h: torch.Tensor, b: StepBatch, cache) -> torch.Tensor:
+        if isinstance(cache, tuple):  # (paged rows, recurrent states): this mixer keeps no state
+            cache = cache[0]
         T, H = h.shape[0], self.H
         z = F.linear(h, self.w_in)
-        a, c = self.qr, self.qr + self.rk + self.dr
-        hops.latent_kv_write(z[:, a:c], self.kv_norm, self.eps, b.pos, self.inv_freq, self.rot_dims, cache, b.slots)
-        cq = hops.rmsnorm_cols(z[:, :a], self.q_norm, self.eps, self.qr, h.dtype)
-        q = F.linear(cq, self.w_uq).view(T, H, self.dn + self.dr)
+        a, c = self.q_cols, self.q_cols + self.rk + self.dr
+        hops.latent_kv_write(z[:, a:c], self.kv_norm, self.eps, b.pos, self.inv_freq, self.rot_dims, cache, b.slots,
+                             self.interleaved, self.rot_amp)
+        if self.qr:
+            cq = hops.rmsnorm_cols(z[:, :a], self.q_norm, self.eps, self.qr, h.dtype)
+            q = F.linear(cq, self.w_uq).view(T, H, self.dn + self.dr)
+        else:
+            q = z[:, :a].unflatten(1, (H, self.dn + self.dr))  # a view: rows keep z's pitch
         q_lat = torch.bmm(q[:, :, :self.dn].transpose(0, 1), self.w_uk).transpose(0, 1)  # [T, H, rank]
-        qa = hops.latent_q_assemble(q_lat, q, b.pos, self.inv_freq, self.rot_dims, self.dn)
+        qa = hops.latent_q_assemble(q_lat, q, b.pos, self.inv_freq, self.rot_dims, self.dn, self.interleaved, self.rot_amp)
         outs = []
         if b.Tp:
             outs.append(hops.latent_attention_prefill(qa[:b.Tp], cache, b.p_bt, b.p_cu, b.p_ctx, self.window,
                                                       self.sink, self.scale, self.rk, b.max_q))
         if T > b.Tp:
             outs.append(hops.latent_attention_decode(qa[b.Tp:], cache, b.d_bt, b.d_ctx, self.window, self.sink,
-                                                     self.scale, self.rk))
+                                                     self.scale, self.rk, max_ctx=b.d_max_ctx))
         o_lat = outs[0] if len(outs) == 1 else torch.cat(outs)
         o = torch.bmm(o_lat.transpose(0, 1), self.w_uv.transpose(1, 2)).transpose(0, 1).reshape(T, H * self.dv)
-        return F.linear(hops.sigmoid_gate_mul(o, z[:, c:]), self.w_o)
+        if self.has_gate:
+            o = hops.sigmoid_gate_mul(o, z[:, c:])
+        return F.linear(o, self.w_o)
+
+
+class CausalConv(nn.Module):
+    """A short causal convolution over time on every channel (weights fp32 ``[channels, taps]``):
+    ``y_t = (u_t if residual) + sum_j w[:, j] u_(t - taps + 1 + j)``; the last ``taps - 1`` inputs of a
+    sequence are its state (one fp32 ``[taps - 1, channels]`` entry per state slot)."""
+
+    def __init__(self, channels: int, taps: int, residual: bool, device=None):
+        super().__init__()
+        self.channels, self.taps, self.residual = channels, taps, residual
+        self.weight = nn.Parameter(torch.zeros(channels, taps, device=device, dtype=torch.float32))
+
+    def state_shape(self):
+        return (self.taps - 1, self.channels)
+
+    def forward(self, u: torch.Tensor, b: StepBatch, state: torch.Tensor) -> torch.Tensor:
+        return hops.causal_conv(u, self.weight, state, b.seq_of, b.cu, b.start, b.state, self.residual)
+
+
+class GroupedAttention(nn.Module):
+    """Grouped-query attention (``heads`` query heads over ``kv_heads`` key / value heads; key size
+    ``dim``, value size ``vdim``) with, each optional: ``conv_taps`` short causal convolutions on the
+    projected q, k, v; per-head RMS norm of q and k; rotary on the first ``rot_dims`` entries (YaRN by
+    ``rot_scaling``, neighbour pairs when ``interleaved``); ``rotate_values``: the value of position j
+    is cached turned by ``j * rot_base^(-2m/vdim)`` per pair m and a head's output at position i is
+    turned back by i, so the sum weighs values by their relative position; ``temperature``: a learned
+    per-head factor on the scaled scores; ``chunk``: position i sees j <= i of its own chunk of that
+    many positions only; ``window``; ``sink``: a learned per-head logit that joins the softmax
+    denominator (not scaled, no value).  The cache row of a token is ``[v | k]`` per kv head."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, rot_base: float, rot_dims: int,
+                 scale: float, eps: float, conv_taps: int = 0, rot_scaling: Optional[dict] = None,
+                 interleaved: bool = True, rotate_values: bool = False, temperature: bool = False,
+                 chunk: Optional[int] = None, window: Optional[int] = None, sink: bool = False, device=None, dtype=None):
+        super().__init__()
+        if heads % kv_heads or rot_dims % 2 or rot_dims > dim:
+            raise ValueError("kv heads must divide the heads; rotary dims must be even and fit the head")
+        if rotate_values and (vdim % 2 or not interleaved):
+            raise ValueError("turned values need an even value size and neighbour pairs")
+        self.width, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.rot_dims, self.scale, self.eps, self.interleaved = rot_dims, scale, eps, interleaved
+        self.chunk = int(chunk) if chunk else hops.NO_LIMIT
+        self.window = int(window) if window else hops.NO_LIMIT
+        kw = dict(device=device, dtype=dtype)
+        f32 = dict(device=device, dtype=torch.float32)
+        cols = (heads + kv_heads) * dim + kv_heads * vdim
+        self.w_qkv = nn.Parameter(torch.empty(cols, width, **kw))  # [W_q ; W_k ; W_v]: the input is read once
+        self.w_o = nn.Parameter(torch.empty(width, heads * vdim, **kw))
+        self.conv = CausalConv(cols, conv_taps, residual=False, device=device) if conv_taps else None
+        self.q_norm = nn.Parameter(torch.ones(dim, **f32))
+        self.k_norm = nn.Parameter(torch.ones(dim, **f32))
+        self.temp = nn.Parameter(torch.ones(heads, **f32)) if temperature else None
+        self.sink = nn.Parameter(torch.zeros(heads, **f32)) if sink else None
+        for w in (self.w_qkv, self.w_o):
+            _init(w, 0.02)
+        inv_freq, self.rot_amp = rotary_frequencies(rot_base, rot_dims, rot_scaling, device)
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+        vf = rotary_frequencies(rot_base, vdim, None, device)[0] if rotate_values else None
+        self.register_buffer("v_freq", vf, persistent=False)
+
+    cache_kind = "latent"  # a paged pool of rows
+
+    @property
+    def cache_row(self) -> int:
+        return self.G * (self.dv + self.dk)
+
+    def state_shapes(self):
+        return [self.conv.state_shape()] if self.conv is not None else []
+
+    def step(self, h: torch.Tensor, b: StepBatch, cache) -> torch.Tensor:
+        rows, states = cache
+        T = h.shape[0]
+        z = F.linear(h, self.w_qkv)
+        if self.conv is not None:
+            z = self.conv(z, b, states[0])
+        q = hops.attn_qkv_prep(z, self.H, self.G, self.dk, self.dv, self.q_norm, self.k_norm, self.eps, b.pos,
+                               self.inv_freq, self.rot_dims, self.interleaved, self.rot_amp, self.v_freq, rows, b.slots)
+        opt = dict(groups=self.G, koff=self.dv, chunk=self.chunk, hscale=self.temp, ofreq=self.v_freq)
+        outs = []
+        if b.Tp:
+            outs.append(hops.latent_attention_prefill(q[:b.Tp], rows, b.p_bt, b.p_cu, b.p_ctx, self.window, self.sink,
+                                                      self.scale, self.dv, b.max_q, **opt))
+        if T > b.Tp:
+            outs.append(hops.latent_attention_decode(q[b.Tp:], rows, b.d_bt, b.d_ctx, self.window, self.sink, self.scale,
+                                                     self.dv, max_ctx=b.d_max_ctx, **opt))
+        o = outs[0] if len(outs) == 1 else torch.cat(outs)
+        return F.linear(o.reshape(T, self.H * self.dv), self.w_o)
+
+
+class ClampedGLU(nn.Module):
+    """Gated feed-forward with clamped branches: ``g = min(W_gate h, limit)``, ``u = clamp(W_up h,
+    -limit, limit)``, ``W_down (g sigmoid(alpha g) (u + 1))``; gate and up are one weight."""
+
+    def __init__(self, width: int, ff: int, limit: float, alpha: float = 1.702, device=None, dtype=None):
+        super().__init__()
+        self.ff, self.limit, self.alpha = ff, float(limit), float(alpha)
+        self.w_gu = nn.Parameter(torch.empty(2 * ff, width, device=device, dtype=dtype))
+        self.w_down = nn.Parameter(torch.empty(width, ff, device=device, dtype=dtype))
+        _init(self.w_gu, 0.02)
+        _init(self.w_down, 0.02)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return F.linear(hops.clamped_glu(F.linear(h, self.w_gu), self.limit, self.alpha), self.w_down)
 
 
 class MLSTM(nn.Module):

@@ -45,5 +45,14 @@ def _register_builtin() -> None:
 
     register(lenitar.ARCHITECTURE, Family(lenitar.LenitarConfig, build, lenitar.load_lenitar))
 
+    from . import dumalix
+
+    def build_dumalix(cfg, device=None, dtype=torch.bfloat16, seed=None):
+        if seed is not None:
+            torch.manual_seed(seed)
+        return dumalix.DumalixLM(cfg, device=device, dtype=dtype)
+
+    register(dumalix.ARCHITECTURE, Family(dumalix.DumalixConfig, build_dumalix, dumalix.load_dumalix))
+
 
 _register_builtin()

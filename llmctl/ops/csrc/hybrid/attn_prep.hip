@@ -1,0 +1,115 @@
+// Query / key / value preparation of grouped-query attention over a paged row cache.
+//
+// Input z [T, H*dk + G*dk + G*dv] = [q | k | v] of a step's packed tokens.  Per token:
+//   q, k   per-head RMS norm over dk (weight shared by the heads), then rotary on the first rot_dims
+//          entries of every head: pairs are neighbours (2i, 2i+1) or halves (i, i + rot_dims/2),
+//          angle = position * freq[i] in fp32, cos and sin times ``amp``;
+//   v      optionally turned the same way over all of dv by position * vfreq[m] (the attention
+//          kernel turns the head's weighted sum back by the query's position);
+//   k, v   written to the token's cache row of kv head g: [v (dv) | k (dk)]; q returned [T, H, dk].
+// One workgroup per token, one wave per head slot in turn; all arithmetic fp32.
+#include "hybrid_common.h"
+
+namespace llmctl_hybrid {
+
+// element index of pair p's two members
+__device__ __forceinline__ void pair_idx(int p, int dims, bool inter, int& i0, int& i1) {
+  if (inter) {
+    i0 = 2 * p;
+    i1 = 2 * p + 1;
+  } else {
+    i0 = p;
+    i1 = p + dims / 2;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict__ z, int64_t z_stride, const float* __restrict__ qn,
+                                                            const float* __restrict__ kn, const int* __restrict__ pos,
+                                                            const float* __restrict__ freq, const float* __restrict__ vfreq,
+                                                            T* __restrict__ q_out, T* __restrict__ cache,
+                                                            const int64_t* __restrict__ slots, int H, int G, int dk, int dv,
+                                                            int rot_dims, int inter, float amp, float eps) {
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float p = (float)pos[t];
+  const int64_t slot = slots[t];
+  const int rs = dv + dk;
+  const T* zr = z + t * z_stride;
+  for (int hs = wave; hs < H + 2 * G; hs += 4) {
+    if (hs < H + G) {  // a query or key head: norm, rotary
+      const bool is_q = hs < H;
+      const T* x = zr + (int64_t)hs * dk;  // k heads follow the q heads at the same pitch
+      const float* nw = is_q ? qn : kn;
+      T* out;
+      if (is_q) out = q_out + (t * H + hs) * dk;
+      else if (slot >= 0) out = cache + (slot * G + (hs - H)) * rs + dv;
+      else continue;
+      float ss = 0.f;
+      for (int c = lane; c < dk; c += 64) {
+        const float v = ldf(x + c);
+        ss += v * v;
+      }
+      const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)dk + eps);
+      for (int pr = lane; pr < rot_dims / 2; pr += 64) {
+        int i0, i1;
+        pair_idx(pr, rot_dims, inter, i0, i1);
+        float s, c;
+        sincosf(p * freq[pr], &s, &c);
+        s *= amp;
+        c *= amp;
+        const float a = ldf(x + i0) * rstd * nw[i0], b = ldf(x + i1) * rstd * nw[i1];
+        stf(out + i0, a * c - b * s);
+        stf(out + i1, b * c + a * s);
+      }
+      for (int c = rot_dims + lane; c < dk; c += 64) stf(out + c, ldf(x + c) * rstd * nw[c]);
+    } else {  // a value head
+      if (slot < 0) continue;
+      const int g = hs - H - G;
+      const T* x = zr + (int64_t)(H + G) * dk + (int64_t)g * dv;
+      T* out = cache + (slot * G + g) * rs;
+      if (vfreq != nullptr) {
+        for (int pr = lane; pr < dv / 2; pr += 64) {
+          int i0, i1;
+          pair_idx(pr, dv, inter, i0, i1);
+          float s, c;
+          sincosf(p * vfreq[pr], &s, &c);
+          const float a = ldf(x + i0), b = ldf(x + i1);
+          stf(out + i0, a * c - b * s);
+          stf(out + i1, b * c + a * s);
+        }
+      } else {
+        for (int c = lane; c < dv; c += 64) stf(out + c, ldf(x + c));
+      }
+    }
+  }
+}
+
+at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, int64_t dv, const at::Tensor& q_norm,
+                         const at::Tensor& k_norm, double eps, const at::Tensor& pos, const at::Tensor& freq, int64_t rot_dims,
+                         bool interleaved, double amp, const c10::optional<at::Tensor>& vfreq, at::Tensor cache, const at::Tensor& slots) {
+  check_rows(z, "z");
+  const int64_t T = z.size(0);
+  HYB_CHECK(H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && dv >= 1 && z.size(1) == (H + G) * dk + G * dv, "z: [T, H*dk + G*dk + G*dv]");
+  auto f32v = [](const at::Tensor& t, int64_t n) { return t.is_cuda() && t.is_contiguous() && t.scalar_type() == at::kFloat && t.numel() == n; };
+  HYB_CHECK(f32v(q_norm, dk) && f32v(k_norm, dk), "q / k norm weights: fp32 [dk]");
+  HYB_CHECK(rot_dims % 2 == 0 && rot_dims >= 0 && rot_dims <= dk && f32v(freq, rot_dims / 2), "rotary: even dims <= dk, fp32 frequencies [dims/2]");
+  if (vfreq.has_value()) HYB_CHECK(dv % 2 == 0 && f32v(*vfreq, dv / 2), "value rotation: even dv, fp32 frequencies [dv/2]");
+  HYB_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == G * (dv + dk) && cache.scalar_type() == z.scalar_type(),
+            "cache: contiguous [blocks, block_size, G * (dv + dk)] of the activation dtype");
+  HYB_CHECK(pos.is_cuda() && pos.is_contiguous() && pos.scalar_type() == at::kInt && pos.numel() == T && slots.is_cuda() && slots.is_contiguous() &&
+                slots.scalar_type() == at::kLong && slots.numel() == T, "pos int32 [T], slots int64 [T]");
+  c10::DeviceGuard guard(z.device());
+  at::Tensor q = at::empty({T, H, dk}, z.options());
+  if (T == 0) return q;
+  dispatch_act(z, [&](auto* tag) {
+    using Tt = std::remove_pointer_t<decltype(tag)>;
+    attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), 256, 0, cur_stream()>>>(
+        (const Tt*)z.data_ptr(), z.stride(0), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), pos.data_ptr<int>(), freq.data_ptr<float>(),
+        vfreq.has_value() ? vfreq->data_ptr<float>() : nullptr, (Tt*)q.data_ptr(), (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)H,
+        (int)G, (int)dk, (int)dv, (int)rot_dims, interleaved ? 1 : 0, (float)amp, (float)eps);
+  });
+  return q;
+}
+
+}  // namespace llmctl_hybrid

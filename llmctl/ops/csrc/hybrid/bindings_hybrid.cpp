@@ -13,13 +13,27 @@ at::Tensor sigmoid_gate_mul(const at::Tensor& o, const at::Tensor& g);
 at::Tensor swiglu_any(const at::Tensor& gu);
 at::Tensor headnorm_gate(const at::Tensor& o, const at::Tensor& w, const at::Tensor& g, double eps, bool out_bf16);
 void latent_kv_write(const at::Tensor& dkv, const at::Tensor& norm_w, double eps, const at::Tensor& pos, const at::Tensor& inv_freq,
-                     int64_t rot_dims, at::Tensor cache, const at::Tensor& slots);
+                     int64_t rot_dims, at::Tensor cache, const at::Tensor& slots, bool interleaved, double amp);
 at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const at::Tensor& pos, const at::Tensor& inv_freq,
-                             int64_t rot_dims, int64_t dn);
+                             int64_t rot_dims, int64_t dn, bool interleaved, double amp);
 at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& cu,
-                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q, bool mfma);
+                               const at::Tensor& ctx, int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk,
+                               int64_t max_q, bool mfma, int64_t groups, int64_t koff, int64_t chunk,
+                               const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq);
 at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx,
-                              int64_t window, const at::Tensor& sink, double scale, int64_t rk, bool mfma);
+                              int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk, bool mfma, int64_t groups,
+                              int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
+                              int64_t max_ctx);
+std::tuple<at::Tensor, at::Tensor> add_rmsnorm2_f32_(at::Tensor x, const c10::optional<at::Tensor>& a, const c10::optional<at::Tensor>& b,
+                                                     const at::Tensor& w1, const c10::optional<at::Tensor>& w2, double eps, bool one_plus,
+                                                     bool out_bf16);
+void residual_add_act_(at::Tensor x, const at::Tensor& a, const c10::optional<at::Tensor>& b);
+at::Tensor clamped_glu(const at::Tensor& gu, double limit, double alpha);
+at::Tensor causal_conv(const at::Tensor& u, const at::Tensor& w, at::Tensor state, const at::Tensor& seq_of, const at::Tensor& cu,
+                       const at::Tensor& start, const at::Tensor& sslot, bool add_input);
+at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, int64_t dv, const at::Tensor& q_norm,
+                         const at::Tensor& k_norm, double eps, const at::Tensor& pos, const at::Tensor& freq, int64_t rot_dims,
+                         bool interleaved, double amp, const c10::optional<at::Tensor>& vfreq, at::Tensor cache, const at::Tensor& slots);
 at::Tensor mlstm_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& gates, const at::Tensor& b_i,
                       const at::Tensor& b_f, double cap, double qscale, at::Tensor S, at::Tensor n, at::Tensor m,
                       const at::Tensor& slots, const at::Tensor& cu, const at::Tensor& start, bool slab,
@@ -38,10 +52,15 @@ TORCH_LIBRARY(llmctl_hybrid, m) {
   m.def("sigmoid_gate_mul(Tensor o, Tensor g) -> Tensor");
   m.def("swiglu_any(Tensor gu) -> Tensor");
   m.def("headnorm_gate(Tensor o, Tensor w, Tensor g, float eps, bool out_bf16) -> Tensor");
-  m.def("latent_kv_write(Tensor dkv, Tensor norm_w, float eps, Tensor pos, Tensor inv_freq, int rot_dims, Tensor(a!) cache, Tensor slots) -> ()");
-  m.def("latent_q_assemble(Tensor q_lat, Tensor q, Tensor pos, Tensor inv_freq, int rot_dims, int dn) -> Tensor");
-  m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor sink, float scale, int rk, int max_q, bool mfma=True) -> Tensor");
-  m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor sink, float scale, int rk, bool mfma=True) -> Tensor");
+  m.def("latent_kv_write(Tensor dkv, Tensor norm_w, float eps, Tensor pos, Tensor inv_freq, int rot_dims, Tensor(a!) cache, Tensor slots, bool interleaved=False, float amp=1.0) -> ()");
+  m.def("latent_q_assemble(Tensor q_lat, Tensor q, Tensor pos, Tensor inv_freq, int rot_dims, int dn, bool interleaved=False, float amp=1.0) -> Tensor");
+  m.def("latent_attn_prefill(Tensor qa, Tensor cache, Tensor bt, Tensor cu, Tensor ctx, int window, Tensor? sink, float scale, int rk, int max_q, bool mfma=True, int groups=1, int koff=0, int chunk=1073741824, Tensor? hscale=None, Tensor? ofreq=None) -> Tensor");
+  m.def("latent_attn_decode(Tensor qa, Tensor cache, Tensor bt, Tensor ctx, int window, Tensor? sink, float scale, int rk, bool mfma=True, int groups=1, int koff=0, int chunk=1073741824, Tensor? hscale=None, Tensor? ofreq=None, int max_ctx=0) -> Tensor");
+  m.def("add_rmsnorm2_f32_(Tensor(a!) x, Tensor? a, Tensor? b, Tensor w1, Tensor? w2, float eps, bool one_plus, bool out_bf16) -> (Tensor, Tensor)");
+  m.def("residual_add_act_(Tensor(a!) x, Tensor a, Tensor? b) -> ()");
+  m.def("clamped_glu(Tensor gu, float limit, float alpha) -> Tensor");
+  m.def("causal_conv(Tensor u, Tensor w, Tensor(a!) state, Tensor seq_of, Tensor cu, Tensor start, Tensor sslot, bool add_input) -> Tensor");
+  m.def("attn_qkv_prep(Tensor z, int H, int G, int dk, int dv, Tensor q_norm, Tensor k_norm, float eps, Tensor pos, Tensor freq, int rot_dims, bool interleaved, float amp, Tensor? vfreq, Tensor(a!) cache, Tensor slots) -> Tensor");
   m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start, bool slab=False, Tensor(d!)? fsum=None, bool write_out=True) -> Tensor");
   m.def("mlstm_chunk_combine(Tensor S, Tensor n, Tensor m, Tensor slots, Tensor start, Tensor base, Tensor locS, Tensor locn, Tensor locm, Tensor fsum, Tensor(a!) iS, Tensor(b!) in_, Tensor(c!) im) -> ()");
   m.def("group_topk_router(Tensor logits, int top, int groups, int keep) -> (Tensor, Tensor)");
@@ -59,6 +78,11 @@ TORCH_LIBRARY_IMPL(llmctl_hybrid, CUDA, m) {
   m.impl("latent_q_assemble", &llmctl_hybrid::latent_q_assemble);
   m.impl("latent_attn_prefill", &llmctl_hybrid::latent_attn_prefill);
   m.impl("latent_attn_decode", &llmctl_hybrid::latent_attn_decode);
+  m.impl("add_rmsnorm2_f32_", &llmctl_hybrid::add_rmsnorm2_f32_);
+  m.impl("residual_add_act_", &llmctl_hybrid::residual_add_act_);
+  m.impl("clamped_glu", &llmctl_hybrid::clamped_glu);
+  m.impl("causal_conv", &llmctl_hybrid::causal_conv);
+  m.impl("attn_qkv_prep", &llmctl_hybrid::attn_qkv_prep);
   m.impl("mlstm_scan", &llmctl_hybrid::mlstm_scan);
   m.impl("mlstm_chunk_combine", &llmctl_hybrid::mlstm_chunk_combine);
   m.impl("group_topk_router", &llmctl_hybrid::group_topk_router);

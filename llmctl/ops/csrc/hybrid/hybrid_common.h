@@ -64,4 +64,16 @@ inline void check_rows(const at::Tensor& t, const char* name) {
   HYB_CHECK(t.is_cuda() && t.dim() == 2 && (t.size(1) == 1 || t.stride(1) == 1), name, ": 2-D GPU tensor with unit column stride");
 }
 
+// Optional parts of attention over a paged row cache (latent_attn*.hip).  A cache row of a token holds
+// ``groups`` sub-rows of equal width; a sub-row's first ``rk`` entries are the value and the entries
+// from ``koff`` on the key.  Query head h reads sub-row h / (H / groups).
+struct RowAttnOpts {
+  int64_t groups = 1;
+  int64_t koff = 0;
+  int64_t chunk = (int64_t)1 << 30;  // position i sees j only if i / chunk == j / chunk
+  const float* hscale = nullptr;      // [H] a factor on every head's scores
+  const float* ofreq = nullptr;       // [rk / 2] turn the output's neighbour pairs back by -position * ofreq
+  int64_t max_ctx = 0;                // the longest context of the step, if the host knows it (sizes decode splits)
+};
+
 }  // namespace llmctl_hybrid

@@ -18,7 +18,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
                                                               const int* __restrict__ pos, const float* __restrict__ inv_freq,
                                                               T* __restrict__ cache, const int64_t* __restrict__ slots, int rk,
-                                                              int dr, int rot_dims, float eps) {
+                                                              int dr, int rot_dims, float eps, int inter, float amp) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const int64_t slot = slots[t];
@@ -37,18 +37,21 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restric
   for (int i = threadIdx.x; i < half; i += 256) {
     float s, c;
     sincosf(p * inv_freq[i], &s, &c);
-    const float u = ldf(xr + rk + i), v = ldf(xr + rk + i + half);
-    stf(out + rk + i, u * c - v * s);
-    stf(out + rk + i + half, v * c + u * s);
+    s *= amp;
+    c *= amp;
+    const int i0 = inter ? 2 * i : i, i1 = inter ? 2 * i + 1 : i + half;  // neighbours or halves
+    const float u = ldf(xr + rk + i0), v = ldf(xr + rk + i1);
+    stf(out + rk + i0, u * c - v * s);
+    stf(out + rk + i1, v * c + u * s);
   }
   for (int i = rot_dims + threadIdx.x; i < dr; i += 256) stf(out + rk + i, ldf(xr + rk + i));
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void latent_q_assemble_kernel(const T* __restrict__ ql, int64_t ql_st, int64_t ql_sh,
-                                                                const T* __restrict__ q, const int* __restrict__ pos,
+                                                                const T* __restrict__ q, int64_t q_st, const int* __restrict__ pos,
                                                                 const float* __restrict__ inv_freq, T* __restrict__ qa, int H,
-                                                                int rk, int dn, int dr, int rot_dims) {
+                                                                int rk, int dn, int dr, int rot_dims, int inter, float amp) {
   const int64_t t = blockIdx.x;
   const int R = rk + dr, half = rot_dims / 2;
   const float p = (float)pos[t];
@@ -60,63 +63,96 @@ __global__ __launch_bounds__(256) void latent_q_assemble_kernel(const T* __restr
     const int h = i / half, c = i - h * half;
     float s, co;
     sincosf(p * inv_freq[c], &s, &co);
-    const T* qr = q + (t * H + h) * (int64_t)(dn + dr) + dn;
-    const float u = ldf(qr + c), v = ldf(qr + c + half);
-    stf(qa + (t * H + h) * R + rk + c, u * co - v * s);
-    stf(qa + (t * H + h) * R + rk + c + half, v * co + u * s);
+    s *= amp;
+    co *= amp;
+    const T* qr = q + t * q_st + h * (int64_t)(dn + dr) + dn;
+    const int i0 = inter ? 2 * c : c, i1 = inter ? 2 * c + 1 : c + half;
+    const float u = ldf(qr + i0), v = ldf(qr + i1);
+    stf(qa + (t * H + h) * R + rk + i0, u * co - v * s);
+    stf(qa + (t * H + h) * R + rk + i1, v * co + u * s);
   }
   const int rest = dr - rot_dims;
   for (int i = threadIdx.x; i < H * rest; i += 256) {
     const int h = i / rest, c = rot_dims + (i - h * rest);
-    qa[(t * H + h) * R + rk + c] = q[(t * H + h) * (int64_t)(dn + dr) + dn + c];
+    qa[(t * H + h) * R + rk + c] = q[t * q_st + h * (int64_t)(dn + dr) + dn + c];
   }
 }
 
 // ---------------------------------------------------------------------------------------- prefill
+// Attention over a paged row cache in its general form (RowAttnOpts): the token's cache row holds G
+// sub-rows of width rs, one per kv group; a sub-row's entries [koff, koff + R) are the key and its
+// first rk entries the value (latent attention: G = 1, koff = 0, R = rs).
+struct GenArgs {
+  const int* bt;
+  const int* ctx;
+  const float* sink;    // nullptr: none
+  const float* hscale;  // nullptr: 1
+  const float* ofreq;   // nullptr: the output is not turned back
+  int bt_stride, H, R, rk, bs, window, chunk, G, rs, koff;
+  float scale;
+};
+
+__device__ __forceinline__ int first_visible(int p, int window, int chunk) { return max(max(p - window + 1, (p / chunk) * chunk), 0); }
+
 // grid (q tiles of 64, sequences, heads * value tiles); one wave per block, lane = query.
 template <typename T, int VT>
-__global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __restrict__ qa, const T* __restrict__ cache,
-                                                                 const int* __restrict__ bt, int bt_stride, const int* __restrict__ cu,
-                                                                 const int* __restrict__ ctx, const float* __restrict__ sink,
-                                                                 T* __restrict__ out, int H, int R, int rk, int bs, int window,
-                                                                 float scale, int nvt) {
+__global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __restrict__ qa, const T* __restrict__ cache, const int* __restrict__ cu,
+                                                                 T* __restrict__ out, GenArgs g, int nvt) {
   extern __shared__ float qT[];  // [R][64]
   const int n = blockIdx.y;
   const int h = blockIdx.z / nvt, v0 = (blockIdx.z % nvt) * VT;
+  const int H = g.H, R = g.R, rk = g.rk, bs = g.bs;
   const int a = cu[n], qlen = cu[n + 1] - a;
   const int q0 = blockIdx.x * 64;
   if (q0 >= qlen) return;
   const int lane = threadIdx.x;
-  const int p0 = ctx[n] - qlen;  // position of the sequence's first query row
+  const int p0 = g.ctx[n] - qlen;  // position of the sequence's first query row
   const bool live = q0 + lane < qlen;
   const int qp = p0 + q0 + lane;
   const int64_t qrow = ((int64_t)(a + q0 + (live ? lane : 0)) * H + h) * R;
   for (int d = 0; d < R; ++d) qT[d * 64 + lane] = live ? ldf(qa + qrow + d) : 0.f;
   const int last = p0 + min(q0 + 63, qlen - 1);
-  int j0 = p0 + q0 - window + 1;
-  if (j0 < 0) j0 = 0;
-  float m = sink[h], l = 1.0f;  // the sink: exp(sink - m) with m = sink
+  const int j0 = first_visible(p0 + q0, g.window, g.chunk);
+  const int lo = first_visible(qp, g.window, g.chunk);
+  const float scale = g.scale * (g.hscale != nullptr ? g.hscale[h] : 1.0f);
+  float m = -INFINITY, l = 0.f;
+  if (g.sink != nullptr) {  // the sink: exp(sink - m) with m = sink
+    m = g.sink[h];
+    l = 1.0f;
+  }
   float acc[VT];
 #pragma unroll
   for (int i = 0; i < VT; ++i) acc[i] = 0.f;
-  const int* btn = bt + (int64_t)n * bt_stride;
+  const int* btn = g.bt + (int64_t)n * g.bt_stride;
+  const int grp = h / (H / g.G);
   for (int j = j0; j <= last; ++j) {
-    const T* row = cache + ((int64_t)btn[j / bs] * bs + j % bs) * R;
+    const T* row = cache + (((int64_t)btn[j / bs] * bs + j % bs) * g.G + grp) * g.rs;
+    const T* key = row + g.koff;
     float s = 0.f;
-    for (int d = 0; d < R; ++d) s += qT[d * 64 + lane] * ldf(row + d);
+    for (int d = 0; d < R; ++d) s += qT[d * 64 + lane] * ldf(key + d);
     s *= scale;
-    const int dist = qp - j;
-    if (live && dist >= 0 && dist < window) {
+    if (live && j <= qp && j >= lo) {
       const float mn = fmaxf(m, s);
-      const float corr = expf(m - mn), p = expf(s - mn);
+      const float corr = expf(m - mn), p = expf(s - mn);  // m = -inf before the first key: corr = 0
       l = l * corr + p;
 #pragma unroll
-      for (int i = 0; i < VT; ++i) acc[i] = acc[i] * corr + p * ldf(row + min(v0 + i, R - 1));
+      for (int i = 0; i < VT; ++i) acc[i] = acc[i] * corr + p * ldf(row + min(v0 + i, rk - 1));
       m = mn;
     }
   }
   if (!live) return;
   const float inv = 1.0f / l;
+  if (g.ofreq != nullptr) {  // neighbour pairs (2m, 2m + 1) turned back by the query's position
+#pragma unroll
+    for (int i = 0; i < VT; i += 2)
+      if (v0 + i + 1 < rk) {
+        float sn, cs;
+        sincosf((float)qp * g.ofreq[(v0 + i) >> 1], &sn, &cs);
+        const float u = acc[i], w = acc[i + 1];
+        acc[i] = u * cs + w * sn;
+        acc[i + 1] = w * cs - u * sn;
+      }
+  }
   T* o = out + ((int64_t)(a + q0 + lane) * H + h) * rk;
 #pragma unroll
   for (int i = 0; i < VT; ++i)
@@ -126,11 +162,10 @@ __global__ __launch_bounds__(64) void latent_attn_prefill_kernel(const T* __rest
 // ----------------------------------------------------------------------------------------- decode
 // grid (sequences, heads); 4 waves, each takes chunks of 64 keys (one key per lane for the score).
 template <typename T, int NA>
-__global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __restrict__ qa, const T* __restrict__ cache,
-                                                                 const int* __restrict__ bt, int bt_stride, const int* __restrict__ ctx,
-                                                                 const float* __restrict__ sink, T* __restrict__ out, int H, int R,
-                                                                 int rk, int bs, int window, float scale) {
+__global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __restrict__ qa, const T* __restrict__ cache, T* __restrict__ out,
+                                                                 GenArgs g) {
   extern __shared__ float sm[];
+  const int H = g.H, R = g.R, rk = g.rk, bs = g.bs;
   float* qs = sm;                                   // [R]
   float* pw = qs + R + (R & 1);                     // [4][64]; the padding keeps ro 8-byte aligned
   int64_t* ro = reinterpret_cast<int64_t*>(pw + 256);  // [4][64]
@@ -138,13 +173,15 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
   float* ac = ml + 8;                               // [4][rk]
   const int n = blockIdx.x, h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int len = ctx[n];
-  const int lo = max(0, len - window);
+  const int len = g.ctx[n];
+  const int lo = first_visible(len - 1, g.window, g.chunk);
   const int nk = len - lo;
   const T* qr = qa + ((int64_t)n * H + h) * R;
   for (int d = threadIdx.x; d < R; d += 256) qs[d] = ldf(qr + d);
   __syncthreads();
-  const int* btn = bt + (int64_t)n * bt_stride;
+  const int* btn = g.bt + (int64_t)n * g.bt_stride;
+  const int grp = h / (H / g.G);
+  const float scale = g.scale * (g.hscale != nullptr ? g.hscale[h] : 1.0f);
   float m = -INFINITY, l = 0.f;
   float acc[NA];
 #pragma unroll
@@ -155,10 +192,10 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
     int64_t slot = 0;
     float s = -INFINITY;
     if (ok) {
-      slot = (int64_t)btn[j / bs] * bs + j % bs;
-      const T* row = cache + slot * R;
+      slot = ((int64_t)btn[j / bs] * bs + j % bs) * g.G + grp;
+      const T* key = cache + slot * g.rs + g.koff;
       float d0 = 0.f;
-      for (int d = 0; d < R; ++d) d0 += qs[d] * ldf(row + d);
+      for (int d = 0; d < R; ++d) d0 += qs[d] * ldf(key + d);
       s = d0 * scale;
     }
     const float mn = fmaxf(m, wave_max(s));  // at least one key of the chunk is valid: finite
@@ -174,7 +211,7 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
     for (int i = 0; i < NA; ++i) acc[i] *= corr;
     for (int jj = 0; jj < cnt; ++jj) {
       const float pj = pw[wave * 64 + jj];
-      const T* row = cache + ro[wave * 64 + jj] * R;
+      const T* row = cache + ro[wave * 64 + jj] * g.rs;
 #pragma unroll
       for (int i = 0; i < NA; ++i) {
         const int d = lane + 64 * i;
@@ -193,11 +230,10 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
     if (d < rk) ac[wave * rk + d] = acc[i];
   }
   __syncthreads();
-  const float sk = sink[h];
-  float M = sk;
+  float M = g.sink != nullptr ? g.sink[h] : -INFINITY;
 #pragma unroll
   for (int w = 0; w < 4; ++w) M = fmaxf(M, ml[w * 2]);
-  float L = expf(sk - M);
+  float L = g.sink != nullptr ? expf(g.sink[h] - M) : 0.f;
   float f[4];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
@@ -209,32 +245,44 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) v += ac[w * rk + d] * f[w];
+    if (g.ofreq != nullptr && (d ^ 1) < rk) {  // turned back together with its pair partner d ^ 1
+      float u = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) u += ac[w * rk + (d ^ 1)] * f[w];
+      float sn, cs;
+      sincosf((float)(len - 1) * g.ofreq[d >> 1], &sn, &cs);
+      v = (d & 1) ? v * cs - u * sn : v * cs + u * sn;
+    }
     stf(o + d, v / L);
   }
 }
 
 // latent_attn_mfma.hip: the matrix-core form for bf16 shapes that fit it
-bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk);
+bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff);
 void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor* cu, const at::Tensor& ctx,
-                      int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out);
+                      int64_t window, const float* sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out, const RowAttnOpts& x);
 
 // ------------------------------------------------------------------------------------------ host
 static void check_cache(const at::Tensor& cache, const at::Tensor& like, int64_t R) {
   HYB_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R && cache.scalar_type() == like.scalar_type(),
-            "cache: contiguous [blocks, block_size, rank + rot] of the activation dtype");
+            "cache: contiguous [blocks, block_size, row width] of the activation dtype");
 }
 
 static void check_i32(const at::Tensor& t, const char* name) {
   HYB_CHECK(t.is_cuda() && t.is_contiguous() && t.scalar_type() == at::kInt, name, ": contiguous int32 GPU tensor");
 }
 
+static bool f32_vec(const at::Tensor& t, int64_t n) {
+  return t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous() && t.numel() == n;
+}
+
 void latent_kv_write(const at::Tensor& dkv, const at::Tensor& norm_w, double eps, const at::Tensor& pos, const at::Tensor& inv_freq,
-                     int64_t rot_dims, at::Tensor cache, const at::Tensor& slots) {
+                     int64_t rot_dims, at::Tensor cache, const at::Tensor& slots, bool interleaved, double amp) {
   check_rows(dkv, "dkv");
   const int64_t T = dkv.size(0), R = dkv.size(1), rk = norm_w.numel();
   HYB_CHECK(rk >= 1 && rk <= R && norm_w.scalar_type() == at::kFloat && norm_w.is_contiguous(), "norm weight: fp32 [rank]");
   const int64_t dr = R - rk;
-  HYB_CHECK(rot_dims % 2 == 0 && rot_dims <= dr && inv_freq.numel() == rot_dims / 2 && inv_freq.scalar_type() == at::kFloat && inv_freq.is_cuda() && inv_freq.is_contiguous(), "rotary: even dims <= rot part, fp32 inverse frequencies [dims/2]");
+  HYB_CHECK(rot_dims % 2 == 0 && rot_dims <= dr && f32_vec(inv_freq, rot_dims / 2), "rotary: even dims <= rot part, fp32 inverse frequencies [dims/2]");
   check_cache(cache, dkv, R);
   check_i32(pos, "pos");
   HYB_CHECK(pos.numel() == T && slots.is_cuda() && slots.is_contiguous() && slots.scalar_type() == at::kLong && slots.numel() == T, "pos int32 [T], slots int64 [T]");
@@ -244,17 +292,17 @@ void latent_kv_write(const at::Tensor& dkv, const at::Tensor& norm_w, double eps
     using Tt = std::remove_pointer_t<decltype(tag)>;
     latent_kv_write_kernel<Tt><<<dim3((unsigned)T), 256, 0, cur_stream()>>>(
         (const Tt*)dkv.data_ptr(), dkv.stride(0), norm_w.data_ptr<float>(), pos.data_ptr<int>(), inv_freq.data_ptr<float>(),
-        (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)rk, (int)dr, (int)rot_dims, (float)eps);
+        (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)rk, (int)dr, (int)rot_dims, (float)eps, interleaved ? 1 : 0, (float)amp);
   });
 }
 
 at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const at::Tensor& pos, const at::Tensor& inv_freq,
-                             int64_t rot_dims, int64_t dn) {
-  HYB_CHECK(q.is_cuda() && q.is_contiguous() && q.dim() == 3, "q: contiguous [T, H, dn + rot]");
+                             int64_t rot_dims, int64_t dn, bool interleaved, double amp) {
+  HYB_CHECK(q.is_cuda() && q.dim() == 3 && (q.size(2) == 1 || q.stride(2) == 1) && q.stride(1) == q.size(2), "q: [T, H, dn + rot], heads back to back");
   const int64_t T = q.size(0), H = q.size(1), dr = q.size(2) - dn;
   HYB_CHECK(q_lat.is_cuda() && q_lat.dim() == 3 && q_lat.size(0) == T && q_lat.size(1) == H && (q_lat.size(2) == 1 || q_lat.stride(2) == 1) && q_lat.scalar_type() == q.scalar_type(), "q_lat: [T, H, rank], unit last stride, q's dtype");
   const int64_t rk = q_lat.size(2);
-  HYB_CHECK(dr >= 0 && rot_dims % 2 == 0 && rot_dims <= dr && inv_freq.numel() == rot_dims / 2 && inv_freq.scalar_type() == at::kFloat && inv_freq.is_cuda() && inv_freq.is_contiguous(), "rotary: even dims <= rot part");
+  HYB_CHECK(dr >= 0 && rot_dims % 2 == 0 && rot_dims <= dr && f32_vec(inv_freq, rot_dims / 2), "rotary: even dims <= rot part");
   check_i32(pos, "pos");
   HYB_CHECK(pos.numel() == T, "pos: int32 [T]");
   c10::DeviceGuard guard(q.device());
@@ -263,31 +311,79 @@ at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const
   dispatch_act(q, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
     latent_q_assemble_kernel<Tt><<<dim3((unsigned)T), 256, 0, cur_stream()>>>(
-        (const Tt*)q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1), (const Tt*)q.data_ptr(), pos.data_ptr<int>(),
-        inv_freq.data_ptr<float>(), (Tt*)qa.data_ptr(), (int)H, (int)rk, (int)dn, (int)dr, (int)rot_dims);
+        (const Tt*)q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1), (const Tt*)q.data_ptr(), q.stride(0), pos.data_ptr<int>(),
+        inv_freq.data_ptr<float>(), (Tt*)qa.data_ptr(), (int)H, (int)rk, (int)dn, (int)dr, (int)rot_dims, interleaved ? 1 : 0, (float)amp);
   });
   return qa;
 }
 
+// The optional tensors of the general form, checked; returns the kernels' view of them.
+static RowAttnOpts row_opts(const at::Tensor& qa, const at::Tensor& cache, int64_t rk, const c10::optional<at::Tensor>& sink, int64_t groups,
+                            int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
+                            int64_t max_ctx, const float** sink_p) {
+  const int64_t H = qa.size(1), R = qa.size(2);
+  HYB_CHECK(groups >= 1 && H % groups == 0 && cache.size(2) % groups == 0, "kv groups must divide the heads and the cache row");
+  const int64_t rs = cache.size(2) / groups;
+  HYB_CHECK(koff >= 0 && koff + R <= rs && rk >= 1 && rk <= rs, "key [koff, koff + R) and value [0, rk) must lie inside a sub-row");
+  HYB_CHECK(chunk >= 1, "chunk >= 1");
+  if (sink.has_value()) HYB_CHECK(f32_vec(*sink, H), "sink: fp32 [H]");
+  if (hscale.has_value()) HYB_CHECK(f32_vec(*hscale, H), "head scale: fp32 [H]");
+  if (ofreq.has_value()) HYB_CHECK(rk % 2 == 0 && f32_vec(*ofreq, rk / 2), "output turn: even value width, fp32 frequencies [rk / 2]");
+  *sink_p = sink.has_value() ? sink->data_ptr<float>() : nullptr;
+  RowAttnOpts x;
+  x.groups = groups;
+  x.koff = koff;
+  x.chunk = std::min<int64_t>(chunk, (int64_t)1 << 30);
+  x.hscale = hscale.has_value() ? hscale->data_ptr<float>() : nullptr;
+  x.ofreq = ofreq.has_value() ? ofreq->data_ptr<float>() : nullptr;
+  x.max_ctx = max_ctx;
+  return x;
+}
+
+static GenArgs gen_args(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx, const float* sink,
+                        int64_t window, double scale, int64_t rk, const RowAttnOpts& x) {
+  GenArgs g;
+  g.bt = bt.data_ptr<int>();
+  g.ctx = ctx.data_ptr<int>();
+  g.sink = sink;
+  g.hscale = x.hscale;
+  g.ofreq = x.ofreq;
+  g.bt_stride = (int)bt.size(1);
+  g.H = (int)qa.size(1);
+  g.R = (int)qa.size(2);
+  g.rk = (int)rk;
+  g.bs = (int)cache.size(1);
+  g.window = (int)window;
+  g.chunk = (int)x.chunk;
+  g.G = (int)x.groups;
+  g.rs = (int)(cache.size(2) / x.groups);
+  g.koff = (int)x.koff;
+  g.scale = (float)scale;
+  return g;
+}
+
 at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& cu,
-                               const at::Tensor& ctx, int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q,
-                               bool mfma) {
+                               const at::Tensor& ctx, int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk,
+                               int64_t max_q, bool mfma, int64_t groups, int64_t koff, int64_t chunk,
+                               const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [T, H, R]");
   const int64_t T = qa.size(0), H = qa.size(1), R = qa.size(2);
-  check_cache(cache, qa, R);
+  check_cache(cache, qa, cache.size(2));
   check_i32(bt, "block tables");
   check_i32(cu, "cu");
   check_i32(ctx, "ctx");
   const int64_t ns = ctx.numel();
   HYB_CHECK(bt.dim() == 2 && bt.size(0) == ns && cu.numel() == ns + 1, "block tables [n, max_blocks], cu [n + 1], ctx [n]");
-  HYB_CHECK(sink.is_cuda() && sink.scalar_type() == at::kFloat && sink.is_contiguous() && sink.numel() == H, "sink: fp32 [H]");
-  HYB_CHECK(rk >= 1 && rk <= R && window >= 1 && max_q >= 1, "rank <= R, window >= 1, max_q >= 1");
-  HYB_CHECK((size_t)R * 64 * sizeof(float) <= 160 * 1024, "rank + rot too wide for the query tile in LDS");
+  HYB_CHECK(window >= 1 && max_q >= 1, "window >= 1, max_q >= 1");
+  window = std::min<int64_t>(window, (int64_t)1 << 30);
+  const float* sink_p;
+  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, 0, &sink_p);
+  HYB_CHECK((size_t)R * 64 * sizeof(float) <= 160 * 1024, "key too wide for the query tile in LDS");
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({T, H, rk}, qa.options());
   if (T == 0 || ns == 0) return out;
-  if (mfma && latent_attn_mfma_ok(qa, rk)) {
-    latent_attn_mfma(qa, cache, bt, &cu, ctx, window, sink, scale, rk, max_q, out);
+  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff)) {
+    latent_attn_mfma(qa, cache, bt, &cu, ctx, window, sink_p, scale, rk, max_q, out, x);
     return out;
   }
   const int VT = rk <= 32 ? 32 : (rk <= 64 ? 64 : 128);
@@ -295,13 +391,12 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
   HYB_CHECK(H * nvt <= 65535 && ns <= 65535, "grid too large");
   dim3 grid((unsigned)((max_q + 63) / 64), (unsigned)ns, (unsigned)(H * nvt));
   const size_t lds = (size_t)R * 64 * sizeof(float);
+  const GenArgs g = gen_args(qa, cache, bt, ctx, sink_p, window, scale, rk, x);
   dispatch_act(qa, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
     auto launch = [&](auto kern) {
       if (lds > 64 * 1024) HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
-      kern<<<grid, 64, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), bt.data_ptr<int>(), (int)bt.size(1),
-                                           cu.data_ptr<int>(), ctx.data_ptr<int>(), sink.data_ptr<float>(), (Tt*)out.data_ptr(), (int)H,
-                                           (int)R, (int)rk, (int)cache.size(1), (int)window, (float)scale, nvt);
+      kern<<<grid, 64, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), cu.data_ptr<int>(), (Tt*)out.data_ptr(), g, nvt);
     };
     if (VT == 32) launch(latent_attn_prefill_kernel<Tt, 32>);
     else if (VT == 64) launch(latent_attn_prefill_kernel<Tt, 64>);
@@ -311,35 +406,38 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
 }
 
 at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor& ctx,
-                              int64_t window, const at::Tensor& sink, double scale, int64_t rk, bool mfma) {
+                              int64_t window, const c10::optional<at::Tensor>& sink, double scale, int64_t rk, bool mfma, int64_t groups,
+                              int64_t koff, int64_t chunk, const c10::optional<at::Tensor>& hscale, const c10::optional<at::Tensor>& ofreq,
+                              int64_t max_ctx) {
   HYB_CHECK(qa.is_cuda() && qa.is_contiguous() && qa.dim() == 3, "qa: contiguous [n, H, R]");
   const int64_t ns = qa.size(0), H = qa.size(1), R = qa.size(2);
-  check_cache(cache, qa, R);
+  check_cache(cache, qa, cache.size(2));
   check_i32(bt, "block tables");
   check_i32(ctx, "ctx");
   HYB_CHECK(bt.dim() == 2 && bt.size(0) == ns && ctx.numel() == ns, "block tables [n, max_blocks], ctx [n]");
-  HYB_CHECK(sink.is_cuda() && sink.scalar_type() == at::kFloat && sink.is_contiguous() && sink.numel() == H, "sink: fp32 [H]");
-  HYB_CHECK(rk >= 1 && rk <= R && window >= 1, "rank <= R, window >= 1");
+  HYB_CHECK(window >= 1, "window >= 1");
+  window = std::min<int64_t>(window, (int64_t)1 << 30);
+  const float* sink_p;
+  const RowAttnOpts x = row_opts(qa, cache, rk, sink, groups, koff, chunk, hscale, ofreq, max_ctx, &sink_p);
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({ns, H, rk}, qa.options());
   if (ns == 0) return out;
-  if (mfma && latent_attn_mfma_ok(qa, rk)) {
-    latent_attn_mfma(qa, cache, bt, nullptr, ctx, window, sink, scale, rk, 1, out);
+  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff)) {
+    latent_attn_mfma(qa, cache, bt, nullptr, ctx, window, sink_p, scale, rk, 1, out, x);
     return out;
   }
-  HYB_CHECK(rk <= 512, "generic decode kernel: rank <= 512");
+  HYB_CHECK(rk <= 512, "generic decode kernel: value width <= 512");
   const int64_t Rp = R + (R & 1);  // keeps the int64 array 8-byte aligned
   const size_t lds = (size_t)(Rp + 256) * 4 + 256 * 8 + 8 * 4 + (size_t)4 * rk * 4;
-  HYB_CHECK(lds <= 64 * 1024 && H <= 65535, "rank + rot too wide");
+  HYB_CHECK(lds <= 64 * 1024 && H <= 65535, "key / value too wide");
   dim3 grid((unsigned)ns, (unsigned)H);
+  const GenArgs g = gen_args(qa, cache, bt, ctx, sink_p, window, scale, rk, x);
   dispatch_act(qa, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
     if (rk <= 128)
-      latent_attn_decode_kernel<Tt, 2><<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), bt.data_ptr<int>(),
-          (int)bt.size(1), ctx.data_ptr<int>(), sink.data_ptr<float>(), (Tt*)out.data_ptr(), (int)H, (int)R, (int)rk, (int)cache.size(1), (int)window, (float)scale);
+      latent_attn_decode_kernel<Tt, 2><<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), (Tt*)out.data_ptr(), g);
     else
-      latent_attn_decode_kernel<Tt, 8><<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), bt.data_ptr<int>(),
-          (int)bt.size(1), ctx.data_ptr<int>(), sink.data_ptr<float>(), (Tt*)out.data_ptr(), (int)H, (int)R, (int)rk, (int)cache.size(1), (int)window, (float)scale);
+      latent_attn_decode_kernel<Tt, 8><<<grid, 256, lds, cur_stream()>>>((const Tt*)qa.data_ptr(), (const Tt*)cache.data_ptr(), (Tt*)out.data_ptr(), g);
   });
   return out;
 }

@@ -34,8 +34,11 @@ struct LArgs {
   const int* bt;
   const int* cu;   // nullptr: one query row per sequence (decode)
   const int* ctx;
-  const float* sink;
+  const float* sink;    // nullptr: no sink
+  const float* hscale;  // nullptr or a factor on every head's scores
+  const float* ofreq;   // nullptr, or [rk / 2]: the output's neighbour pairs are turned back by -position * ofreq
   int H, R, rk, bs, maxb, window, HB, nvt;
+  int G, rs, koff, chunk, hpg;  // kv groups, row width, key's first column, chunk mask size, head tiles per group
   float scale_log2;
   // decode rows with the key range split over blockIdx.x (few sequences would otherwise leave the chip
   // idle): each split writes its unnormalised fp32 output and (running maximum, denominator) here
@@ -57,6 +60,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int r = lane & 31, hh = lane >> 5;
   const int n = blockIdx.y;
   const int hg = blockIdx.z / a.nvt, v0 = (blockIdx.z % a.nvt) * (NDB * 32);
+  const int P = a.H / a.G;                       // query heads per kv group
+  const int grp = hg / a.hpg, hsub = (hg % a.hpg) * a.HB;  // this workgroup's kv group, its first head inside it
   const int q_begin = a.cu ? a.cu[n] : n;
   const int qlen = a.cu ? a.cu[n + 1] - q_begin : 1;
   const int HB = a.HB, TB = 128 / HB;
@@ -66,9 +71,9 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int ctx = a.ctx[n];
   const int pos0 = ctx - qlen;
   const int row = wave * 32 + r;
-  const int my_tok = tok0 + row / HB, my_head = hg * HB + row % HB;
-  const bool valid = my_tok < qlen && my_head < a.H;
-  const int tokc = min(my_tok, qlen - 1), headc = min(my_head, a.H - 1);
+  const int my_tok = tok0 + row / HB, my_head = grp * P + hsub + row % HB;
+  const bool valid = my_tok < qlen && hsub + row % HB < P;
+  const int tokc = min(my_tok, qlen - 1), headc = grp * P + min(hsub + row % HB, P - 1);
   const int my_pos = pos0 + tokc;
   const int* btn = a.bt + (long)n * a.maxb;
 
@@ -88,14 +93,21 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   for (int d = 0; d < NDB; ++d)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
-  float m_i = a.sink[headc] * kLog2e, l_i = 1.0f;  // the sink: one unit of mass at its own logit
-  if (split > 0) {                                 // (counted by the first split only)
+  float m_i = -INFINITY, l_i = 0.f;
+  if (a.sink != nullptr) {  // the sink: one unit of mass at its own logit
+    m_i = a.sink[headc] * kLog2e;
+    l_i = 1.0f;
+  }
+  const float my_scale = a.scale_log2 * (a.hscale != nullptr ? a.hscale[headc] : 1.0f);
+  if (split > 0) {                                 // (the sink is counted by the first split only)
     m_i = -INFINITY;
     l_i = 0.f;
   }
 
   const int first_pos = pos0 + tok0, last_pos = pos0 + min(tok0 + TB, qlen) - 1;
-  int t_lo = max(0, first_pos - a.window + 1) / LKB, t_hi = last_pos / LKB + 1;
+  // the first key a query at position p may see: inside its window and inside its chunk
+  auto first_key = [&](int p) { return max(max(p - a.window + 1, (p / a.chunk) * a.chunk), 0); };
+  int t_lo = first_key(first_pos) / LKB, t_hi = last_pos / LKB + 1;
   if (a.nsplit > 1) {
     const int per = (t_hi - t_lo + a.nsplit - 1) / a.nsplit;
     t_lo += split * per;
@@ -104,7 +116,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   // this wave's rows: positions [w_first, w_last]
   const int w_first = pos0 + min(tok0 + (wave * 32) / HB, qlen - 1);
   const int w_last = pos0 + min(tok0 + (wave * 32 + 31) / HB, qlen - 1);
-  const bool wave_live = tok0 + (wave * 32) / HB < qlen && hg * HB + (HB >= 32 ? (wave * 32) % HB : 0) < a.H;
+  const bool wave_live = tok0 + (wave * 32) / HB < qlen && hsub + (HB >= 32 ? (wave * 32) % HB : 0) < P;
+  const int w_lo = first_key(w_first), my_lo = first_key(my_pos);
 
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const unsigned lds_base = lds_addr(smem);
@@ -129,22 +142,20 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       const int img = g >> 4, rg = g & 15;
       const int krow = rg * 4 + (lane >> 4), chp = lane & 15;
       const long slot = slot_lds[sbuf * LKB + krow];
-      int cb, c;
+      int col;
       if (img < NCB) {
-        cb = img;
-        c = chp ^ swz_row<128>(krow);
+        col = a.koff + (img * 16 + (chp ^ swz_row<128>(krow))) * 8;
       } else {
-        cb = v0 / 128 + (img - NCB);
-        c = chp ^ swz_tr<128>(krow);
+        col = ((v0 / 128 + (img - NCB)) * 16 + (chp ^ swz_tr<128>(krow))) * 8;
       }
-      const int col = min((cb * 16 + c) * 8, a.R - 8);
-      dma16(a.cache + slot * a.R + col, lds_base + (unsigned)(img * LIMG + rg * 1024));
+      col = min(col, a.rs - 8);
+      dma16(a.cache + (slot * a.G + grp) * a.rs + col, lds_base + (unsigned)(img * LIMG + rg * 1024));
     }
     if (t + 1 < t_hi) load_slots(t + 1, sbuf ^ 1);
     vm_wait<0>();
     __syncthreads();
     const int kv0 = t * LKB;
-    if (!wave_live || kv0 > w_last || kv0 + LKB - 1 < w_first - a.window + 1) continue;
+    if (!wave_live || kv0 > w_last || kv0 + LKB - 1 < w_lo) continue;
 
     f32x16 s[2];
 #pragma unroll
@@ -162,9 +173,9 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        float x = s[kb][i] * a.scale_log2;
+        float x = s[kb][i] * my_scale;
         const int key = kv0 + kb * 32 + acc_row(i, hh);
-        if (!valid || key > my_pos || key <= my_pos - a.window || key >= ctx) x = -INFINITY;
+        if (!valid || key > my_pos || key < my_lo || key >= ctx) x = -INFINITY;
         s[kb][i] = x;
         mx = fmaxf(mx, x);
       }
@@ -230,6 +241,16 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       for (int g = 0; g < 4; ++g) {
         const int col = v0 + d * 32 + 8 * g + 4 * hh;
         if (col < a.rk) {
+          if (a.ofreq != nullptr) {  // turn the neighbour pairs (col, col + 1), (col + 2, col + 3) back
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+              float sn, cs;
+              sincosf((float)my_pos * a.ofreq[(col + j) >> 1], &sn, &cs);
+              const float u = o[d][4 * g + j], w = o[d][4 * g + j + 1];
+              o[d][4 * g + j] = u * cs + w * sn;
+              o[d][4 * g + j + 1] = w * cs - u * sn;
+            }
+          }
           unsigned short w4[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) w4[j] = __bfloat16_as_ushort(__float2bfloat16(o[d][4 * g + j] * inv));
@@ -242,8 +263,9 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
 
 // out[row] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M = max_s m_s (splits that saw nothing: m = -inf, l = 0)
 __global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, unsigned short* __restrict__ out,
-                                          int nsplit, int rk) {
+                                          int nsplit, int rk, const float* __restrict__ ofreq, const int* __restrict__ ctx, int H) {
   const long row = blockIdx.x;
+  const float pos = ofreq != nullptr ? (float)(ctx[row / H] - 1) : 0.f;  // one row per sequence: its last position
   const float* ml = ws_ml + row * nsplit * 2;
   float M = -INFINITY;
   for (int s = 0; s < nsplit; ++s) M = fmaxf(M, ml[2 * s]);
@@ -251,9 +273,18 @@ __global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const 
   for (int s = 0; s < nsplit; ++s) L += ml[2 * s + 1] * (ml[2 * s] == -INFINITY ? 0.f : fast_exp2(ml[2 * s] - M));
   const float inv = 1.f / L;
   for (int c = threadIdx.x; c < rk; c += blockDim.x) {
-    float v = 0.f;
+    float v = 0.f, w = 0.f;  // column c and, for the turn back, its pair partner c ^ 1
     for (int s = 0; s < nsplit; ++s)
-      if (ml[2 * s] != -INFINITY) v += ws_o[(row * nsplit + s) * rk + c] * fast_exp2(ml[2 * s] - M);
+      if (ml[2 * s] != -INFINITY) {
+        const float f = fast_exp2(ml[2 * s] - M);
+        v += ws_o[(row * nsplit + s) * rk + c] * f;
+        if (ofreq != nullptr) w += ws_o[(row * nsplit + s) * rk + (c ^ 1)] * f;
+      }
+    if (ofreq != nullptr) {
+      float sn, cs;
+      sincosf(pos * ofreq[c >> 1], &sn, &cs);
+      v = (c & 1) ? v * cs - w * sn : v * cs + w * sn;
+    }
     out[row * rk + c] = __bfloat16_as_ushort(__float2bfloat16(v * inv));
   }
 }
@@ -271,30 +302,33 @@ void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
 }
 }  // namespace
 
-bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk) {
+bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff) {
   const int64_t R = qa.size(2);
-  return qa.scalar_type() == at::kBFloat16 && R % 8 == 0 && rk % 8 == 0 && R <= 640 && qa.size(1) >= 1;
+  return qa.scalar_type() == at::kBFloat16 && R % 8 == 0 && rk % 8 == 0 && rs % 8 == 0 && koff % 8 == 0 && R <= 640 && qa.size(1) >= 1;
 }
 
-// cu: undefined tensor = one row per sequence
+// cu == nullptr: one query row per sequence.  ``x`` carries the optional parts (see RowAttnOpts).
 void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor* cu, const at::Tensor& ctx,
-                      int64_t window, const at::Tensor& sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out) {
+                      int64_t window, const float* sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out, const RowAttnOpts& x) {
   const int64_t H = qa.size(1), R = qa.size(2), ns = ctx.numel();
+  const int64_t G = x.groups, P = H / G, rs = cache.size(2) / G;
   const int ncb = (int)((R + 127) / 128);
   const int ndb = rk <= 64 ? 2 : (rk <= 128 ? 4 : 8);
   const int nvt = (int)((rk + ndb * 32 - 1) / (ndb * 32));
   int HB = 1;
   if (max_q < 64) {
-    while (HB < H && HB < 128) HB *= 2;
+    while (HB < P && HB < 128) HB *= 2;
   }
   const int TB = 128 / HB;
-  const int hgroups = (int)((H + HB - 1) / HB);
+  const int hpg = (int)((P + HB - 1) / HB);  // head tiles per kv group
+  const int hgroups = (int)G * hpg;
   HYB_CHECK(ns <= 65535 && hgroups * nvt <= 65535, "grid too large");
-  // decode rows: split the window's key tiles over workgroups until the launch has a few hundred of them
+  // decode rows: split the visible key tiles over workgroups until the launch has a few hundred of them
   int nsplit = 1;
   at::Tensor ws_o, ws_ml;
   if (cu == nullptr && rk % 4 == 0) {
-    const int tiles = (int)((window + LKB - 1) / LKB) + 1;
+    const int64_t span = std::min<int64_t>(std::min<int64_t>(window, x.chunk), x.max_ctx > 0 ? x.max_ctx : (int64_t)1 << 30);
+    const int tiles = (int)std::min<int64_t>((span + LKB - 1) / LKB + 1, 1 << 20);
     const long blocks = (long)ns * hgroups * nvt;
     while (nsplit < tiles && nsplit < 32 && blocks * nsplit < 512) nsplit *= 2;
     if (nsplit > 1) {
@@ -304,7 +338,8 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
   }
   LArgs a{reinterpret_cast<const unsigned short*>(qa.data_ptr()), reinterpret_cast<const unsigned short*>(cache.data_ptr()),
           reinterpret_cast<unsigned short*>(out.data_ptr()), bt.data_ptr<int>(), cu ? cu->data_ptr<int>() : nullptr, ctx.data_ptr<int>(),
-          sink.data_ptr<float>(), (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
+          sink, x.hscale, x.ofreq, (int)H, (int)R, (int)rk, (int)cache.size(1), (int)bt.size(1), (int)window, HB, nvt,
+          (int)G, (int)rs, (int)x.koff, (int)x.chunk, hpg,
           (float)(scale * 1.4426950408889634), nsplit, nsplit > 1 ? ws_o.data_ptr<float>() : nullptr,
           nsplit > 1 ? ws_ml.data_ptr<float>() : nullptr};
   dim3 grid(nsplit > 1 ? (unsigned)nsplit : (unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
@@ -318,7 +353,8 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
   }
   if (nsplit > 1)
     latent_split_merge_kernel<<<dim3((unsigned)(ns * H)), 128, 0, st>>>(ws_o.data_ptr<float>(), ws_ml.data_ptr<float>(),
-                                                                        reinterpret_cast<unsigned short*>(out.data_ptr()), nsplit, (int)rk);
+                                                                        reinterpret_cast<unsigned short*>(out.data_ptr()), nsplit, (int)rk,
+                                                                        x.ofreq, ctx.data_ptr<int>(), (int)H);
 }
 
 }  // namespace llmctl_hybrid

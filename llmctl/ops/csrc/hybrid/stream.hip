@@ -38,6 +38,50 @@ __global__ __launch_bounds__(NT) void add_layernorm_kernel(float* __restrict__ x
   for (int c = threadIdx.x; c < W; c += NT) stf(h + r * W + c, (xr[c] - mean) * rstd * w[c] + bias[c]);
 }
 
+// x [T, W] fp32 (updated in place when a != nullptr: x += a + b), then up to two RMS norms of the same
+// x (one statistic): h_k = x / sqrt(mean(x^2) + eps) * (plus + w_k); ``plus`` = 1 for weights stored
+// around zero.  A parallel layer's residual update and the two norms its branches read, in one pass.
+template <typename T>
+__global__ __launch_bounds__(NT) void add_rmsnorm2_kernel(float* __restrict__ x, const T* __restrict__ a, int64_t a_stride,
+                                                          const T* __restrict__ b, int64_t b_stride, const float* __restrict__ w1,
+                                                          const float* __restrict__ w2, T* __restrict__ h1, T* __restrict__ h2, int W,
+                                                          float eps, float plus) {
+  __shared__ float red[NW];
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * W;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < W; c += NT) {
+    float v = xr[c];
+    if (a != nullptr) {
+      float d = ldf(a + r * a_stride + c);
+      if (b != nullptr) d += ldf(b + r * b_stride + c);
+      v += d;
+      xr[c] = v;
+    }
+    q += v * v;
+  }
+  if (h1 == nullptr) return;
+  const float rstd = 1.0f / sqrtf(block_sum<NW>(q, red) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += NT) {
+    const float v = xr[c] * rstd;
+    stf(h1 + r * W + c, v * (plus + w1[c]));
+    if (h2 != nullptr) stf(h2 + r * W + c, v * (plus + w2[c]));
+  }
+}
+
+// gu [rows, 2F] = [gate | up] -> g' = min(gate, limit), u' = clamp(up, -limit, limit),
+// y = g' * sigmoid(alpha * g') * (u' + 1)
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ y, int64_t rows, int F, float limit, float alpha) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * F) return;
+  const int64_t r = i / F;
+  const int c = (int)(i - r * F);
+  const float g = fminf(ldf(gu + r * 2 * F + c), limit);
+  const float u = fminf(fmaxf(ldf(gu + r * 2 * F + F + c), -limit), limit);
+  stf(y + i, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void rmsnorm_cols_kernel(const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
                                                           T* __restrict__ y, int n, float eps) {
@@ -191,6 +235,72 @@ at::Tensor swiglu_any(const at::Tensor& gu) {
   dispatch_act(gu, [&](auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
     swiglu_kernel<T><<<dim3((unsigned)((n + 255) / 256)), 256, 0, cur_stream()>>>((const T*)gu.data_ptr(), (T*)y.data_ptr(), gu.size(0), F);
+  });
+  return y;
+}
+
+std::tuple<at::Tensor, at::Tensor> add_rmsnorm2_f32_(at::Tensor x, const c10::optional<at::Tensor>& a, const c10::optional<at::Tensor>& b,
+                                                     const at::Tensor& w1, const c10::optional<at::Tensor>& w2, double eps, bool one_plus,
+                                                     bool out_bf16) {
+  HYB_CHECK(x.is_cuda() && x.dim() == 2 && x.is_contiguous() && x.scalar_type() == at::kFloat, "x: contiguous fp32 [T, W]");
+  const int W = (int)x.size(1);
+  auto okw = [&](const at::Tensor& w) { return w.is_cuda() && w.scalar_type() == at::kFloat && w.numel() == W && w.is_contiguous(); };
+  HYB_CHECK(okw(w1) && (!w2.has_value() || okw(*w2)), "norm weights: fp32 [W]");
+  const at::ScalarType act = out_bf16 ? at::kBFloat16 : at::kFloat;
+  if (a.has_value()) {
+    check_rows(*a, "a");
+    HYB_CHECK(a->sizes() == x.sizes() && a->scalar_type() == act, "a: x's shape, the output dtype");
+    if (b.has_value()) {
+      check_rows(*b, "b");
+      HYB_CHECK(b->sizes() == x.sizes() && b->scalar_type() == act, "b: x's shape, the output dtype");
+    }
+  } else {
+    HYB_CHECK(!b.has_value(), "b without a");
+  }
+  c10::DeviceGuard guard(x.device());
+  at::Tensor h1 = out_like(x, x.sizes(), out_bf16);
+  at::Tensor h2 = w2.has_value() ? out_like(x, x.sizes(), out_bf16) : at::Tensor();
+  if (x.size(0) == 0) return {h1, w2.has_value() ? h2 : h1};
+  dispatch_act(h1, [&](auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    add_rmsnorm2_kernel<T><<<dim3((unsigned)x.size(0)), NT, 0, cur_stream()>>>(
+        x.data_ptr<float>(), a.has_value() ? (const T*)a->data_ptr() : nullptr, a.has_value() ? a->stride(0) : 0,
+        b.has_value() ? (const T*)b->data_ptr() : nullptr, b.has_value() ? b->stride(0) : 0, w1.data_ptr<float>(),
+        w2.has_value() ? w2->data_ptr<float>() : nullptr, (T*)h1.data_ptr(), w2.has_value() ? (T*)h2.data_ptr() : nullptr, W, (float)eps,
+        one_plus ? 1.0f : 0.0f);
+  });
+  return {h1, w2.has_value() ? h2 : h1};
+}
+
+void residual_add_act_(at::Tensor x, const at::Tensor& a, const c10::optional<at::Tensor>& b) {
+  HYB_CHECK(x.is_cuda() && x.dim() == 2 && x.is_contiguous() && x.scalar_type() == at::kFloat, "x: contiguous fp32 [T, W]");
+  check_rows(a, "a");
+  HYB_CHECK(a.sizes() == x.sizes(), "a must have x's shape");
+  if (b.has_value()) {
+    check_rows(*b, "b");
+    HYB_CHECK(b->sizes() == x.sizes() && b->scalar_type() == a.scalar_type(), "b: x's shape, a's dtype");
+  }
+  if (x.size(0) == 0) return;
+  c10::DeviceGuard guard(x.device());
+  dispatch_act(a, [&](auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    add_rmsnorm2_kernel<T><<<dim3((unsigned)x.size(0)), NT, 0, cur_stream()>>>(
+        x.data_ptr<float>(), (const T*)a.data_ptr(), a.stride(0), b.has_value() ? (const T*)b->data_ptr() : nullptr,
+        b.has_value() ? b->stride(0) : 0, nullptr, nullptr, (T*)nullptr, (T*)nullptr, (int)x.size(1), 0.f, 0.f);
+  });
+}
+
+at::Tensor clamped_glu(const at::Tensor& gu, double limit, double alpha) {
+  HYB_CHECK(gu.is_cuda() && gu.is_contiguous() && gu.dim() == 2 && gu.size(1) % 2 == 0, "gu: contiguous [T, 2F]");
+  c10::DeviceGuard guard(gu.device());
+  const int F = (int)(gu.size(1) / 2);
+  at::Tensor y = at::empty({gu.size(0), F}, gu.options());
+  const int64_t n = y.numel();
+  if (n == 0) return y;
+  dispatch_act(gu, [&](auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    clamped_glu_kernel<T><<<dim3((unsigned)((n + 255) / 256)), 256, 0, cur_stream()>>>((const T*)gu.data_ptr(), (T*)y.data_ptr(), gu.size(0), F,
+                                                                                     (float)limit, (float)alpha);
   });
   return y;
 }

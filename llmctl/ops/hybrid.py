@@ -50,39 +50,103 @@ def rmsnorm_cols(x, w, eps: float, n: int, out_dtype):
     return ref.rmsnorm_cols(x, w, eps, n, out_dtype)
 
 
-def latent_kv_write(dkv, norm_w, eps: float, pos, inv_freq, rot_dims: int, cache, slots):
+def latent_kv_write(dkv, norm_w, eps: float, pos, inv_freq, rot_dims: int, cache, slots, interleaved: bool = False,
+                    amp: float = 1.0):
     """The down-projected K/V row ``dkv [T, rank + rot]``: RMS norm of the latent part, rotary on
-    the shared key part, both written to the paged cache row ``[rank | rot]`` at ``slots``."""
+    the shared key part (pairs: halves, or neighbours when ``interleaved``; cos and sin times ``amp``),
+    both written to the paged cache row ``[rank | rot]`` at ``slots``."""
     if use_native(dkv):
-        native_hybrid().latent_kv_write(dkv, norm_w, eps, pos, inv_freq, rot_dims, cache, slots)
+        native_hybrid().latent_kv_write(dkv, norm_w, eps, pos, inv_freq, rot_dims, cache, slots, interleaved, amp)
     else:
-        ref.latent_kv_write(dkv, norm_w, eps, pos, inv_freq, rot_dims, cache, slots)
+        ref.latent_kv_write(dkv, norm_w, eps, pos, inv_freq, rot_dims, cache, slots, interleaved, amp)
 
 
-def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims: int, dn: int):
+def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims: int, dn: int, interleaved: bool = False, amp: float = 1.0):
     """Query rows in the cache's layout: ``[q_lat | rotary(q[..., dn:])]`` per head, where ``q_lat
     [T, H, rank]`` is the unrotated query part carried into the latent space (q W_uk)."""
     if use_native(q):
-        return native_hybrid().latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn)
-    return ref.latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn)
+        return native_hybrid().latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn, interleaved, amp)
+    return ref.latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn, interleaved, amp)
+
+
+NO_LIMIT = 1 << 30  # a window or chunk that never masks
 
 
 def latent_attention_prefill(qa, cache, bt, cu, ctx, window: int, sink, scale: float, rk: int, max_q: int,
-                             mfma: bool = True):
+                             mfma: bool = True, groups: int = 1, koff: int = 0, chunk: int = NO_LIMIT, hscale=None,
+                             ofreq=None):
     """Prompt portions: sequence n's query rows ``[cu[n], cu[n+1])`` end at position ``ctx[n]-1``;
     ``max_q``: the longest portion (sizes the launch).  bf16 shapes that fit run on the matrix cores
-    (``mfma=False`` forces the generic fp32-SIMT kernel, which also serves fp32)."""
+    (``mfma=False`` forces the generic fp32-SIMT kernel, which also serves fp32).
+
+    The general form reads a paged row cache whose token rows hold ``groups`` sub-rows (one per kv
+    group; query head h reads sub-row ``h // (H // groups)``): entries ``[koff, koff + R)`` of a sub-row
+    are the key, its first ``rk`` entries the value.  Latent attention is ``groups=1, koff=0``.  Masks:
+    ``window`` (i - j < window) and ``chunk`` (i // chunk == j // chunk), :data:`NO_LIMIT` for none.
+    ``sink`` (fp32 [H] or None) joins the softmax denominator; ``hscale`` (fp32 [H]) multiplies a head's
+    scores; ``ofreq`` (fp32 [rk/2]) turns the output's neighbour pairs back by ``-position * ofreq``."""
     if use_native(qa):
-        return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q, mfma)
-    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk)
+        return native_hybrid().latent_attn_prefill(qa, cache, bt, cu, ctx, window, sink, scale, rk, max_q, mfma, groups,
+                                                   koff, chunk, hscale, ofreq)
+    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq)
 
 
-def latent_attention_decode(qa, cache, bt, ctx, window: int, sink, scale: float, rk: int, mfma: bool = True):
-    """One query row per sequence, at position ``ctx[n] - 1``."""
+def latent_attention_decode(qa, cache, bt, ctx, window: int, sink, scale: float, rk: int, mfma: bool = True,
+                            groups: int = 1, koff: int = 0, chunk: int = NO_LIMIT, hscale=None, ofreq=None,
+                            max_ctx: int = 0):
+    """One query row per sequence, at position ``ctx[n] - 1`` (options as in the prefill form;
+    ``max_ctx``: the longest context if the host knows it, it sizes the split of the keys)."""
     if use_native(qa):
-        return native_hybrid().latent_attn_decode(qa, cache, bt, ctx, window, sink, scale, rk, mfma)
+        return native_hybrid().latent_attn_decode(qa, cache, bt, ctx, window, sink, scale, rk, mfma, groups, koff, chunk,
+                                                  hscale, ofreq, max_ctx)
     cu = torch.arange(qa.shape[0] + 1, dtype=torch.int32)
-    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk)
+    return ref.latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups, koff, chunk, hscale, ofreq)
+
+
+def add_rmsnorm2_f32_(x, a, b, w1, w2, eps: float, one_plus: bool, out_dtype):
+    """``x += a (+ b)`` in place on the fp32 residual stream (skipped when ``a`` is None), then RMS norms
+    of the same x with weights ``w1`` and (optional) ``w2``: ``x / sqrt(mean(x^2) + eps) * (w + one_plus)``.
+    Returns (h1, h2) in ``out_dtype`` (h2 is h1 when ``w2`` is None)."""
+    if use_native(x):
+        return native_hybrid().add_rmsnorm2_f32_(x, a, b, w1, w2, eps, one_plus, out_dtype == torch.bfloat16)
+    return ref.add_rmsnorm2_f32_(x, a, b, w1, w2, eps, one_plus, out_dtype)
+
+
+def residual_add_act_(x, a, b=None):
+    """``x += a (+ b)`` on the fp32 residual stream, a and b in the activation dtype."""
+    if use_native(x):
+        native_hybrid().residual_add_act_(x, a, b)
+        return x
+    return ref.residual_add_(x, a, b)
+
+
+def clamped_glu(gu, limit: float, alpha: float):
+    """``gu [T, 2F] = [gate | up]`` -> ``g * sigmoid(alpha g) * (u + 1)`` with ``g = min(gate, limit)``,
+    ``u = clamp(up, -limit, limit)``."""
+    if use_native(gu):
+        return native_hybrid().clamped_glu(gu.contiguous(), limit, alpha)
+    return ref.clamped_glu(gu, limit, alpha)
+
+
+def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input: bool):
+    """Short causal convolution over time per channel of the packed rows ``u [T, C]`` (``w`` fp32
+    ``[C, taps]``): ``y_t = (u_t if add_input) + sum_j w[:, j] u_(t - taps + 1 + j)``.  ``state`` (fp32
+    ``[slots, taps - 1, C]``) carries each live sequence's last ``taps - 1`` inputs between steps (read
+    at ``sslot[seq]`` unless the sequence starts at position 0, then updated in place)."""
+    if use_native(u):
+        return native_hybrid().causal_conv(u, w, state, seq_of, cu, start, sslot, add_input)
+    return ref.causal_conv(u, w, state, seq_of, cu, start, sslot, add_input)
+
+
+def attn_qkv_prep(z, H: int, G: int, dk: int, dv: int, q_norm, k_norm, eps: float, pos, freq, rot_dims: int,
+                  interleaved: bool, amp: float, vfreq, cache, slots):
+    """``z [T, H*dk + G*dk + G*dv] = [q | k | v]``: per-head RMS norm (weights fp32 [dk]) and rotary of
+    q and k, optional turn of v over all of dv by ``position * vfreq``; k and v are written to the
+    token's cache row ``[G, dv + dk] = [v | k]`` at ``slots``; returns q ``[T, H, dk]``."""
+    if use_native(z):
+        return native_hybrid().attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp,
+                                             vfreq, cache, slots)
+    return ref.attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp, vfreq, cache, slots)
 
 
 def sigmoid_gate_mul(o, g):

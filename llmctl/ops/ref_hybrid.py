@@ -31,57 +31,139 @@ def rmsnorm_cols(x, w, eps, n, out_dtype):
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
 
 
-def _rotate(x, pos, inv_freq, dims):
-    """x f32 [T, ..., n]: entries [0, dims) rotated in the rotate-half pairing."""
+def _rotate(x, pos, inv_freq, dims, interleaved=False, amp=1.0):
+    """x f32 [T, ..., n]: entries [0, dims) rotated; pairs are halves (i, i + dims/2) or neighbours
+    (2i, 2i + 1); cos and sin are scaled by ``amp``."""
     half = dims // 2
     ang = pos.float()[:, None] * inv_freq.float()[None, :]  # fp32 angles
     shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
-    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    c, s = torch.cos(ang).view(shape) * amp, torch.sin(ang).view(shape) * amp
+    if interleaved:
+        u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+        r = torch.stack([u * c - v * s, v * c + u * s], -1).flatten(-2)
+        return torch.cat([r, x[..., dims:]], -1)
     u, v = x[..., :half], x[..., half:dims]
     return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
 
 
-def latent_kv_write(dkv, norm_w, eps, pos, inv_freq, rot_dims, cache, slots):
+def latent_kv_write(dkv, norm_w, eps, pos, inv_freq, rot_dims, cache, slots, interleaved=False, amp=1.0):
     rk = norm_w.shape[0]
     c = rmsnorm_cols(dkv, norm_w, eps, rk, torch.float32)
-    kr = _rotate(dkv[:, rk:].float(), pos, inv_freq, rot_dims)
+    kr = _rotate(dkv[:, rk:].float(), pos, inv_freq, rot_dims, interleaved, amp)
     row = torch.cat([c, kr], -1).to(cache.dtype)
     ok = slots >= 0
     cache.view(-1, cache.shape[-1])[slots[ok]] = row[ok]
 
 
-def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn):
-    qr = _rotate(q[..., dn:].float(), pos, inv_freq, rot_dims)
+def latent_q_assemble(q_lat, q, pos, inv_freq, rot_dims, dn, interleaved=False, amp=1.0):
+    qr = _rotate(q[..., dn:].float(), pos, inv_freq, rot_dims, interleaved, amp)
     return torch.cat([q_lat.float(), qr], -1).to(q.dtype)
 
 
-def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk):
-    """Sliding-window attention with a sink over the paged latent cache.  Sequence n owns query
-    rows [cu[n], cu[n+1]); its last query sits at position ctx[n] - 1.  Keys and values are cache
-    rows (value = the first ``rk`` entries of the key row), shared by all heads."""
+def latent_attention(qa, cache, bt, cu, ctx, window, sink, scale, rk, groups=1, koff=0, chunk=1 << 30, hscale=None,
+                     ofreq=None):
+    """Attention over a paged row cache.  Sequence n owns query rows [cu[n], cu[n+1]); its last query
+    sits at position ctx[n] - 1.  A token's cache row holds ``groups`` sub-rows; query head h reads
+    sub-row h / (H / groups), whose entries [koff, koff + R) are the key and whose first ``rk`` entries
+    are the value (latent attention: one sub-row, key = the whole row).  Position i sees j <= i inside
+    its window (i - j < window) and its chunk (i // chunk == j // chunk); ``sink`` [H] joins the softmax
+    denominator; ``hscale`` [H] multiplies the scores; ``ofreq`` [rk / 2] turns the output's neighbour
+    pairs back by -position * ofreq."""
     T, H, R = qa.shape
     bs = cache.shape[1]
+    G = groups
+    rs = cache.shape[2] // G
     out = torch.zeros(T, H, rk, dtype=torch.float32)
-    flat = cache.view(-1, R)
+    flat = cache.view(-1, G, rs)
     cu_l, ctx_l = [int(v) for v in cu], [int(v) for v in ctx]
+    hs = hscale.float().view(H, 1, 1) if hscale is not None else 1.0
     for n in range(len(ctx_l)):
         a, b = cu_l[n], cu_l[n + 1]
         if b == a:
             continue
         p0 = ctx_l[n] - (b - a)  # position of the first query row
-        lo = max(0, p0 - window + 1)
+        lo = max(0, p0 - window + 1, (p0 // chunk) * chunk)
         kpos = torch.arange(lo, ctx_l[n])
-        rows = flat[bt[n, (kpos // bs).long()].long() * bs + kpos % bs].float()  # [K, R]
-        s = torch.einsum("thr,kr->htk", qa[a:b].float(), rows) * scale
+        rows = flat[bt[n, (kpos // bs).long()].long() * bs + kpos % bs].float()  # [K, G, rs]
+        rows = rows.repeat_interleave(H // G, 1)  # [K, H, rs]
+        s = torch.einsum("thr,khr->htk", qa[a:b].float(), rows[:, :, koff:koff + R]) * scale * hs
         qpos = torch.arange(p0, ctx_l[n])
         d = qpos[:, None] - kpos[None, :]
-        s = s.masked_fill(~((d >= 0) & (d < window)), float("-inf"))
-        sk = sink.float().view(H, 1, 1)
-        top = torch.maximum(s.max(-1, keepdim=True).values, sk)
+        vis = (d >= 0) & (d < window) & (qpos[:, None] // chunk == kpos[None, :] // chunk)
+        s = s.masked_fill(~vis, float("-inf"))
+        top = s.max(-1, keepdim=True).values
+        if sink is not None:
+            sk = sink.float().view(H, 1, 1)
+            top = torch.maximum(top, sk)
         e = torch.exp(s - top)
-        p = e / (e.sum(-1, keepdim=True) + torch.exp(sk - top))
-        out[a:b] = torch.einsum("htk,kr->thr", p, rows[:, :rk])
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sk - top)
+        o = torch.einsum("htk,khr->thr", e / den, rows[:, :, :rk])
+        if ofreq is not None:
+            o = _rotate(o, -qpos, ofreq, rk, True)
+        out[a:b] = o
     return out.to(qa.dtype)
+
+
+def add_rmsnorm2_f32_(x, a, b, w1, w2, eps, one_plus, out_dtype):
+    if a is not None:
+        x += a.float() + b.float() if b is not None else a.float()
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    plus = 1.0 if one_plus else 0.0
+    h1 = (y * (plus + w1.float())).to(out_dtype)
+    return h1, ((y * (plus + w2.float())).to(out_dtype) if w2 is not None else h1)
+
+
+def clamped_glu(gu, limit, alpha):
+    f = gu.shape[-1] // 2
+    g, u = gu[..., :f].float().clamp(max=limit), gu[..., f:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input):
+    """y_t = (u_t if add_input) + sum_j w[:, j] u_(t - taps + 1 + j) per sequence of the packed rows; the
+    last taps - 1 inputs of a sequence live in ``state[slot]`` ([taps - 1, C], oldest first) between steps
+    and are ignored by a sequence that starts at position 0."""
+    T, C = u.shape
+    taps = w.shape[1]
+    y = torch.zeros(T, C, dtype=torch.float32)
+    cu_l = [int(v) for v in cu]
+    for s in range(len(cu_l) - 1):
+        a, b = cu_l[s], cu_l[s + 1]
+        if a == b:
+            continue
+        slot = int(sslot[s])
+        old = state[slot].clone() if int(start[s]) > 0 else torch.zeros(taps - 1, C)
+        if 0 < int(start[s]) < taps - 1:  # entries of positions before 0
+            old[:taps - 1 - int(start[s])] = 0.0
+        ext = torch.cat([old, u[a:b].float()], 0)
+        n = b - a
+        acc = torch.zeros(n, C)
+        for j in range(taps):
+            acc += ext[j:j + n] * w[:, j].float()
+        y[a:b] = acc + (u[a:b].float() if add_input else 0.0)
+        if taps > 1:
+            state[slot] = ext[-(taps - 1):]
+    return y.to(u.dtype)
+
+
+def attn_qkv_prep(z, H, G, dk, dv, q_norm, k_norm, eps, pos, freq, rot_dims, interleaved, amp, vfreq, cache, slots):
+    """z [T, H*dk + G*dk + G*dv] = [q | k | v]: per-head RMS norm and rotary of q and k, optional turn of
+    v over all of dv; k and v go to the token's cache row [G, dv + dk] = [v | k]; returns q [T, H, dk]."""
+    T = z.shape[0]
+    zf = z.float()
+    q, k = zf[:, :H * dk].view(T, H, dk), zf[:, H * dk:(H + G) * dk].view(T, G, dk)
+    v = zf[:, (H + G) * dk:].view(T, G, dv)
+    unit = lambda x: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    q = _rotate(unit(q) * q_norm.float(), pos, freq, rot_dims, interleaved, amp)
+    k = _rotate(unit(k) * k_norm.float(), pos, freq, rot_dims, interleaved, amp)
+    if vfreq is not None:
+        v = _rotate(v, pos, vfreq, dv, interleaved)
+    row = torch.cat([v, k], -1).reshape(T, G * (dv + dk)).to(cache.dtype)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok]] = row[ok]
+    return q.to(z.dtype)
 
 
 def sigmoid_gate_mul(o, g):

@@ -209,7 +209,9 @@ class HybridCache:
     """The cache of a model whose layers mix differently: per layer either a paged pool of cache rows
     (``("latent", row_width)``: ``[num_blocks, block_size, row_width]``, addressed through the same
     block tables as a K/V cache) or fp32 recurrent-state pools (``("state", [shape, ...])``:
-    ``[num_slots, *shape]`` each, addressed by the sequence's slot).  Layers may differ in size."""
+    ``[num_slots, *shape]`` each, addressed by the sequence's slot), or both (``("rows+state",
+    (row_width, [shape, ...]))``: ``layer(i)`` is ``(rows, (state, ...))``).  Entries may differ in size; a
+    model whose layers run more than once (a looped stack) lists one entry per layer run."""
 
     def __init__(self, kinds, num_blocks: int, block_size: int, num_slots: int, dtype=torch.bfloat16, device=None):
         self.num_blocks, self.block_size, self.num_slots = num_blocks, block_size, num_slots
@@ -220,9 +222,14 @@ class HybridCache:
             elif kind == "state":
                 self._layers.append(tuple(torch.zeros((num_slots,) + tuple(s), dtype=torch.float32, device=device)
                                           for s in spec))
+            elif kind == "rows+state":
+                row, shapes = spec
+                self._layers.append((torch.zeros(num_blocks, block_size, int(row), dtype=dtype, device=device),
+                                     tuple(torch.zeros((num_slots,) + tuple(s), dtype=torch.float32, device=device)
+                                           for s in shapes)))
             else:
                 raise ValueError(f"unknown cache kind {kind!r}")
-        self.has_state = any(k == "state" for k, _ in kinds)
+        self.has_state = any(k == "state" or (k == "rows+state" and len(s[1]) > 0) for k, s in kinds)
         self.slots = StateSlotManager(num_slots) if self.has_state else None
 
     def layer(self, i: int):
@@ -230,12 +237,14 @@ class HybridCache:
 
     @staticmethod
     def bytes_per_block(kinds, block_size: int, dtype_bytes: int) -> int:
-        return max(sum(int(s) for k, s in kinds if k == "latent") * block_size * dtype_bytes, 1)
+        rows = sum(int(s) for k, s in kinds if k == "latent") + sum(int(s[0]) for k, s in kinds if k == "rows+state")
+        return max(rows * block_size * dtype_bytes, 1)
 
     @property
     def nbytes(self) -> int:
-        n = 0
-        for l in self._layers:
-            for t in (l if isinstance(l, tuple) else (l,)):
-                n += t.numel() * t.element_size()
-        return n
+        def size(l):
+            if isinstance(l, tuple):
+                return sum(size(t) for t in l)
+            return l.numel() * l.element_size()
+
+        return sum(size(l) for l in self._layers)

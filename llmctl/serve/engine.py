@@ -158,10 +158,13 @@ class InferenceEngine:
             raise ValueError("hybrid-mixer models keep their cache and weights in the model dtype")
         self._w8 = self._w8_head = self._nf = None
         self.weight_dtype, self.kv_dtype, self.rope = "auto", self.dtype, None
-        kinds = []
-        for layer in self.model.layers:
-            m = layer.mixer
-            kinds.append(("latent", m.cache_row) if m.cache_kind == "latent" else ("state", m.state_shapes()))
+        if hasattr(self.model, "cache_kinds"):  # the model lists its cache entries itself (one per layer run)
+            kinds = self.model.cache_kinds()
+        else:
+            kinds = []
+            for layer in self.model.layers:
+                m = layer.mixer
+                kinds.append(("latent", m.cache_row) if m.cache_kind == "latent" else ("state", m.state_shapes()))
         bs = self.block_size
         if num_kv_blocks is None:
             if self.device.type == "cuda":
@@ -218,11 +221,13 @@ class InferenceEngine:
         start = ([c - (b - a) for a, b, c in zip(p_cu[:-1], p_cu[1:], pp["ctx"])] if Tp else []) + (
             list(dp["positions"]) if Td else [])
         state = (list(pp["state"]) if Tp else []) + (list(dp["state"]) if Td else [])
+        seq_of = np.repeat(np.arange(len(cu) - 1, dtype=np.int32), np.diff(np.asarray(cu, dtype=np.int64)))
         batch = StepBatch(ids=i64(ids), pos=i32(pos), slots=i64(slots), Tp=Tp,
                           p_cu=i32(p_cu) if Tp else None, p_ctx=i32(pp["ctx"]) if Tp else None,
                           p_bt=i32(pp["bt"]) if Tp else None, d_ctx=i32(dp["ctx"]) if Td else None,
                           d_bt=i32(dp["bt"]) if Td else None, cu=i32(cu), start=i32(start), state=i32(state),
-                          max_q=max((b - a for a, b in zip(p_cu[:-1], p_cu[1:])), default=0), cu_host=cu)
+                          max_q=max((b - a for a, b in zip(p_cu[:-1], p_cu[1:])), default=0), cu_host=cu,
+                          seq_of=i32(seq_of), d_max_ctx=int(max(dp["ctx"])) if Td else 0)
         if rows is None:
             rows = (list(pp["last"]) if Tp else []) + list(range(Tp, Tp + Td))
         if count:
