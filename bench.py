@@ -61,20 +61,28 @@ def parse():
                     help="instead of the training benchmark: serving prefill / decode throughput of Lenitar "
                          "configurations beside the routed-expert transformer at equal size (comma-separated "
                          "sizes of llmctl.benchmarks.hybrid.SIZES, or 'all'); one JSON line per size")
+    ap.add_argument("--dumalix-compare", default=None, metavar="SIZES",
+                    help="instead of the training benchmark: serving prefill / decode throughput of Dumalix "
+                         "configurations beside the dense grouped-query transformer at equal size (comma-separated "
+                         "sizes of llmctl.benchmarks.hybrid.DUMALIX_SIZES, or 'all'); one JSON line per size")
     return ap.parse_args()
 
 
 def hybrid_compare(args) -> None:
     from llmctl.benchmarks import hybrid
 
-    names = sorted(hybrid.SIZES) if args.hybrid_compare == "all" else args.hybrid_compare.split(",")
-    for row in hybrid.run(names, device=args.device, steps=args.steps, warmup=args.warmup):
+    if args.dumalix_compare:
+        table, which, family = hybrid.DUMALIX_SIZES, args.dumalix_compare, "dumalix"
+    else:
+        table, which, family = hybrid.SIZES, args.hybrid_compare, "lenitar"
+    names = sorted(table) if which == "all" else which.split(",")
+    for row in hybrid.run(names, device=args.device, steps=args.steps, warmup=args.warmup, family=family):
         print(json.dumps(row), flush=True)
 
 
 def main():
     args = parse()
-    if args.hybrid_compare:
+    if args.hybrid_compare or args.dumalix_compare:
         return hybrid_compare(args)
     import torch
     import torch.distributed as dist

@@ -1,5 +1,7 @@
 """Serving throughput of a Lenitar configuration beside the closest existing model (the routed-expert
-transformer: softmax attention + top-k SwiGLU experts) at equal width, depth, heads and experts.
+transformer: softmax attention + top-k SwiGLU experts) at equal width, depth, heads and experts, and of
+a Dumalix configuration beside the dense transformer (grouped-query softmax attention + SwiGLU) at equal
+width, layer runs, heads, kv heads and feed-forward size.
 
 Both run through the same engine calls: one prompt portion per sequence (``InferenceEngine.prefill``)
 and then one-token decode steps of the whole batch (``InferenceEngine.decode``); random weights,
@@ -21,6 +23,29 @@ SIZES = {
     "medium": dict(width=2048, layers=4, heads=16, experts=8, top=2, ff=1024, window=1024, prompt=2048, batch=16),
     "large": dict(width=4096, layers=4, heads=32, experts=8, top=2, ff=2048, window=1024, prompt=4096, batch=16),
 }
+
+
+# Dumalix: width, layers (every third is chunked grouped-query attention, the others latent attention),
+# loop (start, stop, times), heads of 128, kv heads, feed-forward, chunk, prompt, decode batch
+DUMALIX_SIZES = {
+    "tiny": dict(width=128, layers=3, loop=(1, 3, 2), heads=4, kv_heads=2, head_dim=32, ff=192, chunk=32, prompt=64, batch=2),
+    "small": dict(width=1024, layers=6, loop=(1, 3, 2), heads=8, kv_heads=2, head_dim=128, ff=3072, chunk=1024, prompt=2048, batch=16),
+    "medium": dict(width=2048, layers=6, loop=(1, 3, 2), heads=16, kv_heads=4, head_dim=128, ff=6144, chunk=1024, prompt=2048, batch=16),
+    "large": dict(width=4096, layers=6, loop=(1, 3, 2), heads=32, kv_heads=8, head_dim=128, ff=12288, chunk=2048, prompt=4096, batch=16),
+}
+
+
+def _configs_dumalix(s: Dict):
+    from llmctl.models.config import ModelConfig
+    from llmctl.models.dumalix import dumalix_template
+
+    du = dumalix_template(width=s["width"], layers=s["layers"], heads=s["heads"], kv_heads=s["kv_heads"], vocab=32000, every=3,
+                          ff=s["ff"], chunk=s["chunk"], taps=4, loop=s["loop"], head_dim=s["head_dim"])
+    du.max_position_embeddings = s["prompt"] + 256
+    runs = len(du.runs())
+    tr = ModelConfig(name=f"dense-w{s['width']}-l{runs}", layers=runs, hidden=s["width"], ffn=s["ff"], heads=s["heads"],
+                     kv_heads=s["kv_heads"], vocab_size=32000, max_position_embeddings=s["prompt"] + 256)
+    return du, tr
 
 
 def _configs(s: Dict):
@@ -99,13 +124,20 @@ def _measure(eng, prompt: int, batch: int, steps: int, warmup: int) -> Dict[str,
             "decode_ms": round(dec * 1e3, 3), "decode_tok_s": round(batch / dec, 1)}
 
 
-def run(sizes: List[str], device: str = "auto", steps: int = 5, warmup: int = 2) -> List[Dict]:
+def run(sizes: List[str], device: str = "auto", steps: int = 5, warmup: int = 2, family: str = "lenitar") -> List[Dict]:
     out = []
     for name in sizes:
-        s = SIZES[name]
-        hy, tr = _configs(s)
-        row = {"size": name, **{k: s[k] for k in ("width", "layers", "heads", "experts", "top", "ff", "window", "prompt", "batch")}}
-        for label, cfg in (("lenitar", hy), ("moe_transformer", tr)):
+        if family == "dumalix":
+            s = DUMALIX_SIZES[name]
+            hy, tr = _configs_dumalix(s)
+            row = {"size": name, **s, "layer_runs": len(hy.runs())}
+            pair = (("dumalix", hy), ("dense_transformer", tr))
+        else:
+            s = SIZES[name]
+            hy, tr = _configs(s)
+            row = {"size": name, **{k: s[k] for k in ("width", "layers", "heads", "experts", "top", "ff", "window", "prompt", "batch")}}
+            pair = (("lenitar", hy), ("moe_transformer", tr))
+        for label, cfg in pair:
             eng = _engine(cfg, device, s["prompt"], s["batch"])
             row[label] = _measure(eng, s["prompt"], s["batch"], steps, warmup)
             row[label]["params_m"] = round(sum(p.numel() for p in eng.model.parameters()) / 1e6, 1)

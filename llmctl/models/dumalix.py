@@ -175,7 +175,9 @@ class DumalixLM(nn.Module):
     def dtype(self):
         return self.embed.dtype
 
-    has_recurrent_state = True
+    @property
+    def has_recurrent_state(self) -> bool:
+        return any(len(l.state_shapes()) > 0 for l in self.layers)
 
     def head_weight(self):
         return self.lm_head
