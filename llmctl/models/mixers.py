@@ -168,7 +168,8 @@ class CausalConv(nn.Module):
         return (self.taps - 1, self.channels)
 
     def forward(self, u: torch.Tensor, b: StepBatch, state: torch.Tensor) -> torch.Tensor:
-        return hops.causal_conv(u, self.weight, state, b.seq_of, b.cu, b.start, b.state, self.residual)
+        return hops.causal_conv(u, self.weight, state, b.seq_of, b.cu, b.start, b.state, self.residual,
+                                max_len=max(b.max_q, 1 if u.shape[0] > b.Tp else 0))
 
 
 class GroupedAttention(nn.Module):

@@ -7,7 +7,8 @@
 //   v      optionally turned the same way over all of dv by position * vfreq[m] (the attention
 //          kernel turns the head's weighted sum back by the query's position);
 //   k, v   written to the token's cache row of kv head g: [v (dv) | k (dk)]; q returned [T, H, dk].
-// One workgroup per token, one wave per head slot in turn; all arithmetic fp32.
+// One workgroup per token, one wave per head slot in turn; all arithmetic fp32.  The token's cos / sin
+// (they depend on the position and the pair only) are computed once into LDS and shared by its heads.
 #include "hybrid_common.h"
 
 namespace llmctl_hybrid {
@@ -30,9 +31,24 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict_
                                                             T* __restrict__ q_out, T* __restrict__ cache,
                                                             const int64_t* __restrict__ slots, int H, int G, int dk, int dv,
                                                             int rot_dims, int inter, float amp, float eps) {
+  extern __shared__ float cs_tab[];  // [rot_dims / 2][2] cos, sin (times amp), then [dv / 2][2] for the values
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float p = (float)pos[t];
+  const int nrot = rot_dims / 2, nv = vfreq != nullptr ? dv / 2 : 0;
+  for (int i = threadIdx.x; i < nrot + nv; i += 256) {
+    float s, c;
+    if (i < nrot) {
+      sincosf(p * freq[i], &s, &c);
+      s *= amp;
+      c *= amp;
+    } else {
+      sincosf(p * vfreq[i - nrot], &s, &c);
+    }
+    cs_tab[2 * i] = c;
+    cs_tab[2 * i + 1] = s;
+  }
+  __syncthreads();
   const int64_t slot = slots[t];
   const int rs = dv + dk;
   const T* zr = z + t * z_stride;
@@ -54,10 +70,7 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict_
       for (int pr = lane; pr < rot_dims / 2; pr += 64) {
         int i0, i1;
         pair_idx(pr, rot_dims, inter, i0, i1);
-        float s, c;
-        sincosf(p * freq[pr], &s, &c);
-        s *= amp;
-        c *= amp;
+        const float c = cs_tab[2 * pr], s = cs_tab[2 * pr + 1];
         const float a = ldf(x + i0) * rstd * nw[i0], b = ldf(x + i1) * rstd * nw[i1];
         stf(out + i0, a * c - b * s);
         stf(out + i1, b * c + a * s);
@@ -72,8 +85,7 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict_
         for (int pr = lane; pr < dv / 2; pr += 64) {
           int i0, i1;
           pair_idx(pr, dv, inter, i0, i1);
-          float s, c;
-          sincosf(p * vfreq[pr], &s, &c);
+          const float c = cs_tab[2 * (nrot + pr)], s = cs_tab[2 * (nrot + pr) + 1];
           const float a = ldf(x + i0), b = ldf(x + i1);
           stf(out + i0, a * c - b * s);
           stf(out + i1, b * c + a * s);
@@ -104,7 +116,7 @@ at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, 
   if (T == 0) return q;
   dispatch_act(z, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), 256, 0, cur_stream()>>>(
+    attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), 256, (size_t)(rot_dims + dv) * sizeof(float), cur_stream()>>>(
         (const Tt*)z.data_ptr(), z.stride(0), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), pos.data_ptr<int>(), freq.data_ptr<float>(),
         vfreq.has_value() ? vfreq->data_ptr<float>() : nullptr, (Tt*)q.data_ptr(), (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)H,
         (int)G, (int)dk, (int)dv, (int)rot_dims, interleaved ? 1 : 0, (float)amp, (float)eps);

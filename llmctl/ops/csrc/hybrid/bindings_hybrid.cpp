@@ -30,7 +30,7 @@ std::tuple<at::Tensor, at::Tensor> add_rmsnorm2_f32_(at::Tensor x, const c10::op
 void residual_add_act_(at::Tensor x, const at::Tensor& a, const c10::optional<at::Tensor>& b);
 at::Tensor clamped_glu(const at::Tensor& gu, double limit, double alpha);
 at::Tensor causal_conv(const at::Tensor& u, const at::Tensor& w, at::Tensor state, const at::Tensor& seq_of, const at::Tensor& cu,
-                       const at::Tensor& start, const at::Tensor& sslot, bool add_input);
+                       const at::Tensor& start, const at::Tensor& sslot, bool add_input, int64_t max_len);
 at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, int64_t dv, const at::Tensor& q_norm,
                          const at::Tensor& k_norm, double eps, const at::Tensor& pos, const at::Tensor& freq, int64_t rot_dims,
                          bool interleaved, double amp, const c10::optional<at::Tensor>& vfreq, at::Tensor cache, const at::Tensor& slots);
@@ -59,7 +59,7 @@ TORCH_LIBRARY(llmctl_hybrid, m) {
   m.def("add_rmsnorm2_f32_(Tensor(a!) x, Tensor? a, Tensor? b, Tensor w1, Tensor? w2, float eps, bool one_plus, bool out_bf16) -> (Tensor, Tensor)");
   m.def("residual_add_act_(Tensor(a!) x, Tensor a, Tensor? b) -> ()");
   m.def("clamped_glu(Tensor gu, float limit, float alpha) -> Tensor");
-  m.def("causal_conv(Tensor u, Tensor w, Tensor(a!) state, Tensor seq_of, Tensor cu, Tensor start, Tensor sslot, bool add_input) -> Tensor");
+  m.def("causal_conv(Tensor u, Tensor w, Tensor(a!) state, Tensor seq_of, Tensor cu, Tensor start, Tensor sslot, bool add_input, int max_len=0) -> Tensor");
   m.def("attn_qkv_prep(Tensor z, int H, int G, int dk, int dv, Tensor q_norm, Tensor k_norm, float eps, Tensor pos, Tensor freq, int rot_dims, bool interleaved, float amp, Tensor? vfreq, Tensor(a!) cache, Tensor slots) -> Tensor");
   m.def("mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor gates, Tensor b_i, Tensor b_f, float cap, float qscale, Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor slots, Tensor cu, Tensor start, bool slab=False, Tensor(d!)? fsum=None, bool write_out=True) -> Tensor");
   m.def("mlstm_chunk_combine(Tensor S, Tensor n, Tensor m, Tensor slots, Tensor start, Tensor base, Tensor locS, Tensor locn, Tensor locm, Tensor fsum, Tensor(a!) iS, Tensor(b!) in_, Tensor(c!) im) -> ()");

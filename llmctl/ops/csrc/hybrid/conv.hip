@@ -5,8 +5,12 @@
 // sequence that starts at position 0 ignores what its slot holds.
 //
 //   causal_conv_kernel        one thread per (token, channel); fp32 arithmetic
+//   causal_conv_vec_kernel    the same with 16-byte accesses (8 bf16 / 4 fp32 channels per thread), for
+//                             channel counts and row pitches that allow them
 //   causal_conv_state_kernel  after it (stream order): the slot's new content from the step's rows and,
 //                             for portions shorter than taps - 1, the slot's old content
+//   causal_conv_short_kernel  steps whose portions are all short (decode rows): one thread per (sequence,
+//                             channel) walks the portion's tokens and then writes the slot, in one launch
 #include "hybrid_common.h"
 
 namespace llmctl_hybrid {
@@ -41,6 +45,73 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ 
 }
 
 template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_vec_kernel(const T* __restrict__ u, int64_t u_stride, const float* __restrict__ w,
+                                                              const float* __restrict__ state, const int* __restrict__ seq_of,
+                                                              const int* __restrict__ cu, const int* __restrict__ start,
+                                                              const int* __restrict__ sslot, T* __restrict__ y, int C, int taps,
+                                                              int add_input) {
+  constexpr int N = Vec16<T>::N;
+  const int64_t t = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * N;
+  if (c >= C) return;
+  const int s = seq_of[t];
+  const int li = (int)t - cu[s];
+  const int p0 = start[s];
+  const float* st = state + (int64_t)sslot[s] * (taps - 1) * C;
+  float cur[N], acc[N], v[N];
+  Vec16<T>::load(u + t * u_stride + c, cur);
+#pragma unroll
+  for (int i = 0; i < N; ++i) acc[i] = w[(int64_t)(c + i) * taps + taps - 1] * cur[i];
+  for (int k = 1; k < taps; ++k) {
+    const int i0 = li - k;
+    if (i0 >= 0) {
+      Vec16<T>::load(u + (t - k) * u_stride + c, v);
+    } else if (p0 + i0 >= 0) {
+#pragma unroll
+      for (int i = 0; i < N; i += 4) Vec16<float>::load(st + (int64_t)(taps - 1 + i0) * C + c + i, v + i);
+    } else {
+      continue;
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] += w[(int64_t)(c + i) * taps + taps - 1 - k] * v[i];
+  }
+  if (add_input) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] += cur[i];
+  }
+  Vec16<T>::store(y + t * (int64_t)C + c, acc);
+}
+
+// Portions of at most CONV_SHORT tokens: thread (sequence, channel) keeps the last taps - 1 inputs in
+// registers, walks the portion and writes the slot back; the convolution and the state update are one launch.
+constexpr int CONV_SHORT = 4;
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_short_kernel(const T* __restrict__ u, int64_t u_stride, const float* __restrict__ w,
+                                                                float* __restrict__ state, const int* __restrict__ cu,
+                                                                const int* __restrict__ start, const int* __restrict__ sslot,
+                                                                T* __restrict__ y, int C, int taps, int add_input) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int a = cu[s], n = cu[s + 1] - a;
+  if (n <= 0) return;
+  const int p0 = start[s];
+  float* st = state + (int64_t)sslot[s] * (taps - 1) * C;
+  float h[CONV_MAX_TAPS];  // h[j]: the input taps - 1 - j positions before the current token (h[taps-1] = current)
+  for (int j = 0; j < taps - 1; ++j) h[j] = (p0 - (taps - 1) + j >= 0) ? st[(int64_t)j * C + c] : 0.f;
+  const float* wc = w + (int64_t)c * taps;
+  for (int i = 0; i < n; ++i) {
+    const float cur = ldf(u + (int64_t)(a + i) * u_stride + c);
+    h[taps - 1] = cur;
+    float acc = add_input ? cur : 0.f;
+    for (int j = 0; j < taps; ++j) acc += wc[j] * h[j];
+    stf(y + (int64_t)(a + i) * C + c, acc);
+    for (int j = 0; j < taps - 1; ++j) h[j] = h[j + 1];
+  }
+  for (int j = 0; j < taps - 1; ++j) st[(int64_t)j * C + c] = h[j];
+}
+
+template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_state_kernel(const T* __restrict__ u, int64_t u_stride, float* __restrict__ state,
                                                                 const int* __restrict__ cu, const int* __restrict__ start,
                                                                 const int* __restrict__ sslot, int C, int taps) {
@@ -62,8 +133,9 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(const T* __restr
   }
 }
 
+// max_len: the longest portion of the step if the host knows it (0 = unknown)
 at::Tensor causal_conv(const at::Tensor& u, const at::Tensor& w, at::Tensor state, const at::Tensor& seq_of, const at::Tensor& cu,
-                       const at::Tensor& start, const at::Tensor& sslot, bool add_input) {
+                       const at::Tensor& start, const at::Tensor& sslot, bool add_input, int64_t max_len) {
   check_rows(u, "u");
   const int64_t T = u.size(0), C = u.size(1);
   HYB_CHECK(w.is_cuda() && w.dim() == 2 && w.is_contiguous() && w.scalar_type() == at::kFloat && w.size(0) == C, "w: contiguous fp32 [C, taps]");
@@ -82,9 +154,21 @@ at::Tensor causal_conv(const at::Tensor& u, const at::Tensor& w, at::Tensor stat
   HYB_CHECK(cb <= 65535, "too many channels for one launch");
   dispatch_act(u, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    causal_conv_kernel<Tt><<<dim3((unsigned)T, cb), 256, 0, cur_stream()>>>(
-        (const Tt*)u.data_ptr(), u.stride(0), w.data_ptr<float>(), state.data_ptr<float>(), seq_of.data_ptr<int>(), cu.data_ptr<int>(),
-        start.data_ptr<int>(), sslot.data_ptr<int>(), (Tt*)y.data_ptr(), C, (int)C, (int)taps, add_input ? 1 : 0);
+    if (max_len >= 1 && max_len <= CONV_SHORT) {
+      causal_conv_short_kernel<Tt><<<dim3((unsigned)ns, cb), 256, 0, cur_stream()>>>(
+          (const Tt*)u.data_ptr(), u.stride(0), w.data_ptr<float>(), state.data_ptr<float>(), cu.data_ptr<int>(), start.data_ptr<int>(),
+          sslot.data_ptr<int>(), (Tt*)y.data_ptr(), (int)C, (int)taps, add_input ? 1 : 0);
+      return;
+    }
+    constexpr int N = Vec16<Tt>::N;
+    if (C % 8 == 0 && aligned16<Tt>(u) && reinterpret_cast<uintptr_t>(state.data_ptr()) % 16 == 0)
+      causal_conv_vec_kernel<Tt><<<dim3((unsigned)T, (unsigned)((C / N + 255) / 256)), 256, 0, cur_stream()>>>(
+          (const Tt*)u.data_ptr(), u.stride(0), w.data_ptr<float>(), state.data_ptr<float>(), seq_of.data_ptr<int>(), cu.data_ptr<int>(),
+          start.data_ptr<int>(), sslot.data_ptr<int>(), (Tt*)y.data_ptr(), (int)C, (int)taps, add_input ? 1 : 0);
+    else
+      causal_conv_kernel<Tt><<<dim3((unsigned)T, cb), 256, 0, cur_stream()>>>(
+          (const Tt*)u.data_ptr(), u.stride(0), w.data_ptr<float>(), state.data_ptr<float>(), seq_of.data_ptr<int>(), cu.data_ptr<int>(),
+          start.data_ptr<int>(), sslot.data_ptr<int>(), (Tt*)y.data_ptr(), C, (int)C, (int)taps, add_input ? 1 : 0);
     if (taps > 1)
       causal_conv_state_kernel<Tt><<<dim3((unsigned)ns, cb), 256, 0, cur_stream()>>>(
           (const Tt*)u.data_ptr(), u.stride(0), state.data_ptr<float>(), cu.data_ptr<int>(), start.data_ptr<int>(), sslot.data_ptr<int>(),

@@ -52,19 +52,24 @@ __global__ __launch_bounds__(256) void latent_q_assemble_kernel(const T* __restr
                                                                 const T* __restrict__ q, int64_t q_st, const int* __restrict__ pos,
                                                                 const float* __restrict__ inv_freq, T* __restrict__ qa, int H,
                                                                 int rk, int dn, int dr, int rot_dims, int inter, float amp) {
+  extern __shared__ float cs_tab[];  // the token's [rot_dims / 2][2] cos, sin (times amp), shared by its heads
   const int64_t t = blockIdx.x;
   const int R = rk + dr, half = rot_dims / 2;
   const float p = (float)pos[t];
+  for (int i = threadIdx.x; i < half; i += 256) {
+    float s, co;
+    sincosf(p * inv_freq[i], &s, &co);
+    cs_tab[2 * i] = co * amp;
+    cs_tab[2 * i + 1] = s * amp;
+  }
+  __syncthreads();
   for (int i = threadIdx.x; i < H * rk; i += 256) {
     const int h = i / rk, c = i - h * rk;
     qa[(t * H + h) * R + c] = ql[t * ql_st + h * ql_sh + c];
   }
   for (int i = threadIdx.x; i < H * half; i += 256) {
     const int h = i / half, c = i - h * half;
-    float s, co;
-    sincosf(p * inv_freq[c], &s, &co);
-    s *= amp;
-    co *= amp;
+    const float co = cs_tab[2 * c], s = cs_tab[2 * c + 1];
     const T* qr = q + t * q_st + h * (int64_t)(dn + dr) + dn;
     const int i0 = inter ? 2 * c : c, i1 = inter ? 2 * c + 1 : c + half;
     const float u = ldf(qr + i0), v = ldf(qr + i1);
@@ -258,7 +263,7 @@ __global__ __launch_bounds__(256) void latent_attn_decode_kernel(const T* __rest
 }
 
 // latent_attn_mfma.hip: the matrix-core form for bf16 shapes that fit it
-bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff);
+bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff, bool turn_back);
 void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::Tensor& bt, const at::Tensor* cu, const at::Tensor& ctx,
                       int64_t window, const float* sink, double scale, int64_t rk, int64_t max_q, at::Tensor& out, const RowAttnOpts& x);
 
@@ -310,7 +315,7 @@ at::Tensor latent_q_assemble(const at::Tensor& q_lat, const at::Tensor& q, const
   if (T == 0) return qa;
   dispatch_act(q, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    latent_q_assemble_kernel<Tt><<<dim3((unsigned)T), 256, 0, cur_stream()>>>(
+    latent_q_assemble_kernel<Tt><<<dim3((unsigned)T), 256, (size_t)rot_dims * sizeof(float), cur_stream()>>>(
         (const Tt*)q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1), (const Tt*)q.data_ptr(), q.stride(0), pos.data_ptr<int>(),
         inv_freq.data_ptr<float>(), (Tt*)qa.data_ptr(), (int)H, (int)rk, (int)dn, (int)dr, (int)rot_dims, interleaved ? 1 : 0, (float)amp);
   });
@@ -382,7 +387,7 @@ at::Tensor latent_attn_prefill(const at::Tensor& qa, const at::Tensor& cache, co
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({T, H, rk}, qa.options());
   if (T == 0 || ns == 0) return out;
-  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff)) {
+  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr)) {
     latent_attn_mfma(qa, cache, bt, &cu, ctx, window, sink_p, scale, rk, max_q, out, x);
     return out;
   }
@@ -422,7 +427,7 @@ at::Tensor latent_attn_decode(const at::Tensor& qa, const at::Tensor& cache, con
   c10::DeviceGuard guard(qa.device());
   at::Tensor out = at::empty({ns, H, rk}, qa.options());
   if (ns == 0) return out;
-  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff)) {
+  if (mfma && latent_attn_mfma_ok(qa, rk, cache.size(2) / groups, koff, x.ofreq != nullptr)) {
     latent_attn_mfma(qa, cache, bt, nullptr, ctx, window, sink_p, scale, rk, 1, out, x);
     return out;
   }

@@ -47,13 +47,17 @@ struct LArgs {
   float* ws_ml;  // [rows, nsplit, 2]
 };
 
-template <int NCB, int NDB>
+// ROT: the output's neighbour pairs are turned back by the query's position (a.ofreq); a template flag
+// so that the forms without it keep their register budget
+template <int NCB, int NDB, bool ROT>
 __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   constexpr int NKS = NCB * 8;
   constexpr int NTB = (NDB + 3) / 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* Ks = smem;
-  unsigned char* Vs = smem + NCB * LIMG;
+  // the tile images: one set, or two (the fill of tile t + 1 then runs beside the products of tile t)
+  // where two fit LDS
+  constexpr int BUFB = (NCB + NTB) * LIMG;
+  constexpr bool DB = 2 * BUFB + 1024 <= 160 * 1024;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -122,21 +126,18 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const unsigned lds_base = lds_addr(smem);
   // cache slots of a tile's 64 keys, looked up in the block table one tile ahead (double-buffered)
-  int* slot_lds = reinterpret_cast<int*>(smem + (NCB + NTB) * LIMG);
+  int* slot_lds = reinterpret_cast<int*>(smem + (DB ? 2 : 1) * BUFB);
   auto load_slots = [&](int t, int buf) {
     if (tid < LKB) {
       const int key = min(t * LKB + tid, ctx - 1);
       slot_lds[buf * LKB + tid] = btn[key / a.bs] * a.bs + key % a.bs;
     }
   };
-  if (t_lo < t_hi) load_slots(t_lo, 0);
-  for (int t = t_lo; t < t_hi; ++t) {
-    const int sbuf = (t - t_lo) & 1;
-    __syncthreads();
-    // LDS-DMA fill: every wave instruction moves 4 key rows x 256 B of one image straight from the cache
-    // to LDS (no registers, all pieces of the tile in flight at once); the images' swizzles are applied
-    // to the source chunk.  Keys past the context and columns past R read a valid neighbour instead
-    // (finite data): such keys are masked below and such columns meet zero Q entries or are never stored.
+  // LDS-DMA fill: every wave instruction moves 4 key rows x 256 B of one image straight from the cache
+  // to LDS (no registers, all pieces of the tile in flight at once); the images' swizzles are applied
+  // to the source chunk.  Keys past the context and columns past the row read a valid neighbour instead
+  // (finite data): such keys are masked below and such columns meet zero Q entries or are never stored.
+  auto fill = [&](int sbuf, int ibuf) {
 #pragma unroll 4
     for (int g = wave_u; g < 16 * (NCB + NTB); g += 4) {
       const int img = g >> 4, rg = g & 15;
@@ -149,11 +150,44 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
         col = ((v0 / 128 + (img - NCB)) * 16 + (chp ^ swz_tr<128>(krow))) * 8;
       }
       col = min(col, a.rs - 8);
-      dma16(a.cache + (slot * a.G + grp) * a.rs + col, lds_base + (unsigned)(img * LIMG + rg * 1024));
+      dma16(a.cache + (slot * a.G + grp) * a.rs + col, lds_base + (unsigned)(ibuf * BUFB + img * LIMG + rg * 1024));
     }
-    if (t + 1 < t_hi) load_slots(t + 1, sbuf ^ 1);
-    vm_wait<0>();
-    __syncthreads();
+  };
+  // double-buffered form: the slots of tile t + 2 are requested BEFORE the fill of tile t + 1 is issued and
+  // stored to LDS at the top of the next iteration, so that no wave waits on its own fill in between (a
+  // wave's memory operations complete in order)
+  auto slot_of = [&](int t) {
+    const int key = min(t * LKB + tid, ctx - 1);
+    return btn[key / a.bs] * a.bs + key % a.bs;
+  };
+  int pend = 0;
+  if (t_lo < t_hi) load_slots(t_lo, 0);
+  if constexpr (DB) {
+    if (t_lo < t_hi) {
+      __syncthreads();
+      if (t_lo + 1 < t_hi && tid < LKB) pend = slot_of(t_lo + 1);
+      fill(0, 0);
+    }
+  }
+  for (int t = t_lo; t < t_hi; ++t) {
+    const int sbuf = (t - t_lo) & 1;
+    const unsigned char* Ks = smem + (DB ? sbuf * BUFB : 0);
+    const unsigned char* Vs = Ks + NCB * LIMG;
+    if constexpr (DB) {
+      // tile t was requested one iteration ago.  After the barrier every wave's pieces of it have landed,
+      // every wave is done with tile t - 1 (its images may be overwritten) and the slots of t + 1 are visible
+      if (t + 1 < t_hi && tid < LKB) slot_lds[(sbuf ^ 1) * LKB + tid] = pend;
+      vm_wait<0>();
+      __syncthreads();
+      if (t + 2 < t_hi && tid < LKB) pend = slot_of(t + 2);
+      if (t + 1 < t_hi) fill(sbuf ^ 1, sbuf ^ 1);
+    } else {
+      __syncthreads();
+      fill(sbuf, 0);
+      if (t + 1 < t_hi) load_slots(t + 1, sbuf ^ 1);
+      vm_wait<0>();
+      __syncthreads();
+    }
     const int kv0 = t * LKB;
     if (!wave_live || kv0 > w_last || kv0 + LKB - 1 < w_lo) continue;
 
@@ -241,7 +275,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       for (int g = 0; g < 4; ++g) {
         const int col = v0 + d * 32 + 8 * g + 4 * hh;
         if (col < a.rk) {
-          if (a.ofreq != nullptr) {  // turn the neighbour pairs (col, col + 1), (col + 2, col + 3) back
+          if constexpr (ROT) {  // turn the neighbour pairs (col, col + 1), (col + 2, col + 3) back
 #pragma unroll
             for (int j = 0; j < 4; j += 2) {
               float sn, cs;
@@ -289,22 +323,24 @@ __global__ void latent_split_merge_kernel(const float* __restrict__ ws_o, const 
   }
 }
 
-template <int NCB>
+template <int NCB, bool ROT>
 void launch_ncb(const LArgs& a, int ndb, dim3 grid, hipStream_t st) {
   auto go = [&](auto kern, int NDBv) {
-    const size_t lds = (size_t)(NCB + (NDBv + 3) / 4) * LIMG + 2 * LKB * sizeof(int);
+    const size_t one = (size_t)(NCB + (NDBv + 3) / 4) * LIMG;
+    const size_t lds = (2 * one + 1024 <= 160 * 1024 ? 2 * one : one) + 2 * LKB * sizeof(int);
     HYB_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess, "LDS size");
     kern<<<grid, 256, lds, st>>>(a);
   };
-  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2>, 2);
-  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4>, 4);
-  else go(latent_attn_mfma_kernel<NCB, 8>, 8);
+  if (ndb == 2) go(latent_attn_mfma_kernel<NCB, 2, ROT>, 2);
+  else if (ndb == 4) go(latent_attn_mfma_kernel<NCB, 4, ROT>, 4);
+  else go(latent_attn_mfma_kernel<NCB, 8, ROT>, 8);
 }
 }  // namespace
 
-bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff) {
+// turn_back: the output is to be turned back (RowAttnOpts::ofreq); built for keys up to 256 wide
+bool latent_attn_mfma_ok(const at::Tensor& qa, int64_t rk, int64_t rs, int64_t koff, bool turn_back) {
   const int64_t R = qa.size(2);
-  return qa.scalar_type() == at::kBFloat16 && R % 8 == 0 && rk % 8 == 0 && rs % 8 == 0 && koff % 8 == 0 && R <= 640 && qa.size(1) >= 1;
+  return qa.scalar_type() == at::kBFloat16 && R % 8 == 0 && rk % 8 == 0 && rs % 8 == 0 && koff % 8 == 0 && R <= (turn_back ? 256 : 640) && qa.size(1) >= 1;
 }
 
 // cu == nullptr: one query row per sequence.  ``x`` carries the optional parts (see RowAttnOpts).
@@ -344,12 +380,17 @@ void latent_attn_mfma(const at::Tensor& qa, const at::Tensor& cache, const at::T
           nsplit > 1 ? ws_ml.data_ptr<float>() : nullptr};
   dim3 grid(nsplit > 1 ? (unsigned)nsplit : (unsigned)((max_q + TB - 1) / TB), (unsigned)ns, (unsigned)(hgroups * nvt));
   hipStream_t st = cur_stream();
-  switch (ncb) {
-    case 1: launch_ncb<1>(a, ndb, grid, st); break;
-    case 2: launch_ncb<2>(a, ndb, grid, st); break;
-    case 3: launch_ncb<3>(a, ndb, grid, st); break;
-    case 4: launch_ncb<4>(a, ndb, grid, st); break;
-    default: launch_ncb<5>(a, ndb, grid, st); break;
+  if (x.ofreq != nullptr) {
+    if (ncb == 1) launch_ncb<1, true>(a, ndb, grid, st);
+    else launch_ncb<2, true>(a, ndb, grid, st);
+  } else {
+    switch (ncb) {
+      case 1: launch_ncb<1, false>(a, ndb, grid, st); break;
+      case 2: launch_ncb<2, false>(a, ndb, grid, st); break;
+      case 3: launch_ncb<3, false>(a, ndb, grid, st); break;
+      case 4: launch_ncb<4, false>(a, ndb, grid, st); break;
+      default: launch_ncb<5, false>(a, ndb, grid, st); break;
+    }
   }
   if (nsplit > 1)
     latent_split_merge_kernel<<<dim3((unsigned)(ns * H)), 128, 0, st>>>(ws_o.data_ptr<float>(), ws_ml.data_ptr<float>(),

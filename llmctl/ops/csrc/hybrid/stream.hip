@@ -82,6 +82,26 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ y, 
   stf(y + i, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
 }
 
+// the same with 16-byte accesses (F a multiple of 8, aligned rows): one thread per 8 bf16 / 4 fp32 outputs
+template <typename T>
+__global__ void clamped_glu_vec_kernel(const T* __restrict__ gu, T* __restrict__ y, int64_t rows, int F, float limit, float alpha) {
+  constexpr int N = Vec16<T>::N;
+  const int per = F / N;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * per) return;
+  const int64_t r = i / per;
+  const int c = (int)(i - r * per) * N;
+  float g[N], u[N], o[N];
+  Vec16<T>::load(gu + r * 2 * F + c, g);
+  Vec16<T>::load(gu + r * 2 * F + F + c, u);
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    const float gk = fminf(g[k], limit), uk = fminf(fmaxf(u[k], -limit), limit);
+    o[k] = gk / (1.0f + expf(-alpha * gk)) * (uk + 1.0f);
+  }
+  Vec16<T>::store(y + r * F + c, o);
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void rmsnorm_cols_kernel(const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
                                                           T* __restrict__ y, int n, float eps) {
@@ -299,8 +319,14 @@ at::Tensor clamped_glu(const at::Tensor& gu, double limit, double alpha) {
   if (n == 0) return y;
   dispatch_act(gu, [&](auto* tag) {
     using T = std::remove_pointer_t<decltype(tag)>;
-    clamped_glu_kernel<T><<<dim3((unsigned)((n + 255) / 256)), 256, 0, cur_stream()>>>((const T*)gu.data_ptr(), (T*)y.data_ptr(), gu.size(0), F,
-                                                                                     (float)limit, (float)alpha);
+    if (F % 8 == 0 && aligned16<T>(gu)) {
+      const int64_t nv = n / Vec16<T>::N;
+      clamped_glu_vec_kernel<T><<<dim3((unsigned)((nv + 255) / 256)), 256, 0, cur_stream()>>>((const T*)gu.data_ptr(), (T*)y.data_ptr(), gu.size(0),
+                                                                                            F, (float)limit, (float)alpha);
+    } else {
+      clamped_glu_kernel<T><<<dim3((unsigned)((n + 255) / 256)), 256, 0, cur_stream()>>>((const T*)gu.data_ptr(), (T*)y.data_ptr(), gu.size(0), F,
+                                                                                       (float)limit, (float)alpha);
+    }
   });
   return y;
 }
