@@ -56,6 +56,7 @@ class StepBatch:
     cu_host: Optional[list] = None  # ``cu`` on the host (chunk-parallel scans split long portions)
     seq_of: Optional[torch.Tensor] = None  # int32 [T] index (into cu / start / state) of every row's sequence
     d_max_ctx: int = 0  # the longest context among the decoding sequences
+    fresh: bool = False  # every row belongs to a prompt portion that starts at position 0 (no earlier context)
 
 
 def rotary_frequencies(base: float, dims: int, scaling: Optional[dict] = None, device=None):
@@ -125,6 +126,36 @@ class LatentAttention(nn.Module):
     def state_shapes(self):
         return []
 
+    EXPAND_MIN_TOKENS = 128
+
+    def _expand(self, b: StepBatch) -> bool:
+        """Whole prompts (no earlier context) attend per-head keys and values expanded from the step's own
+        latents when that is the cheaper product: a score then costs dim + rot and a value vdim per head
+        instead of rank + rot and rank.  Steps with earlier context, and decode rows, attend the cached rows."""
+        return (b.fresh and b.Tp >= self.EXPAND_MIN_TOKENS
+                and 2 * self.rk + self.dr > 2 * (self.dn + self.dr + self.dv))
+
+    def _w_uvk(self) -> torch.Tensor:
+        """[W_uv ; W_uk] per head as one weight [H * (vdim + dim), rank] (made once; serving weights are static)."""
+        key = (self.w_uv.data_ptr(), self.w_uv._version, self.w_uk._version)
+        if getattr(self, "_uvk_key", None) != key:
+            self._uvk = torch.cat([self.w_uv.detach(), self.w_uk.detach()], 1).reshape(-1, self.rk).contiguous()
+            self._uvk_key = key
+        return self._uvk
+
+    def _attend_expanded(self, q: torch.Tensor, b: StepBatch, cache: torch.Tensor) -> torch.Tensor:
+        T, H, dn, dr, dv = q.shape[0], self.H, self.dn, self.dr, self.dv
+        lat = cache.view(-1, self.rk + dr).index_select(0, b.slots)  # the rows just written: [latent | rotary key]
+        rows = torch.empty(T, H, dv + dn + dr, device=q.device, dtype=q.dtype)  # per head [v | k | shared rotary key]
+        rows[:, :, :dv + dn] = F.linear(lat[:, :self.rk], self._w_uvk()).view(T, H, dv + dn)
+        rows[:, :, dv + dn:] = lat[:, None, self.rk:]
+        qa = hops.latent_q_assemble(q[:, :, :dn], q, b.pos, self.inv_freq, self.rot_dims, dn, self.interleaved, self.rot_amp)
+        # the step's rows as a cache of one-token pages: sequence n's position j is row p_cu[n] + j
+        bt = (b.p_cu[:-1, None] + torch.arange(b.max_q, device=q.device, dtype=torch.int32)[None, :]).clamp_(max=T - 1)
+        o = hops.latent_attention_prefill(qa, rows.view(T, 1, -1), bt.contiguous(), b.p_cu, b.p_ctx, self.window, self.sink,
+                                          self.scale, dv, b.max_q, groups=H, koff=dv)
+        return o.reshape(T, H * dv)
+
     def step(self, h: torch.Tensor, b: StepBatch, cache) -> torch.Tensor:
         if isinstance(cache, tuple):  # (paged rows, recurrent states): this mixer keeps no state
             cache = cache[0]
@@ -138,6 +169,11 @@ class LatentAttention(nn.Module):
             q = F.linear(cq, self.w_uq).view(T, H, self.dn + self.dr)
         else:
             q = z[:, :a].unflatten(1, (H, self.dn + self.dr))  # a view: rows keep z's pitch
+        if self._expand(b):
+            o = self._attend_expanded(q, b, cache)
+            if self.has_gate:
+                o = hops.sigmoid_gate_mul(o, z[:, c:])
+            return F.linear(o, self.w_o)
         q_lat = torch.bmm(q[:, :, :self.dn].transpose(0, 1), self.w_uk).transpose(0, 1)  # [T, H, rank]
         qa = hops.latent_q_assemble(q_lat, q, b.pos, self.inv_freq, self.rot_dims, self.dn, self.interleaved, self.rot_amp)
         outs = []
@@ -163,12 +199,20 @@ class CausalConv(nn.Module):
         super().__init__()
         self.channels, self.taps, self.residual = channels, taps, residual
         self.weight = nn.Parameter(torch.zeros(channels, taps, device=device, dtype=torch.float32))
+        self._wt, self._wt_key = None, None
 
     def state_shape(self):
         return (self.taps - 1, self.channels)
 
+    def tap_major(self) -> torch.Tensor:
+        """The weights as the kernels read them, ``[taps, channels]`` (made once; serving weights are static)."""
+        w = self.weight
+        if self._wt is None or self._wt_key != (w.data_ptr(), w._version, w.device):
+            self._wt, self._wt_key = w.detach().t().contiguous(), (w.data_ptr(), w._version, w.device)
+        return self._wt
+
     def forward(self, u: torch.Tensor, b: StepBatch, state: torch.Tensor) -> torch.Tensor:
-        return hops.causal_conv(u, self.weight, state, b.seq_of, b.cu, b.start, b.state, self.residual,
+        return hops.causal_conv(u, self.tap_major(), state, b.seq_of, b.cu, b.start, b.state, self.residual,
                                 max_len=max(b.max_q, 1 if u.shape[0] > b.Tp else 0))
 
 

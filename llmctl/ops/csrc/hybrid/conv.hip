@@ -1,6 +1,7 @@
 // Short causal convolution over time on every channel of a step's packed tokens, with the last
 // taps - 1 inputs of each live sequence carried in a slot pool between steps:
-//   y_t = (add_input ? u_t : 0) + sum_j w[c][j] * u_(t - taps + 1 + j),   zeros before position 0.
+//   y_t = (add_input ? u_t : 0) + sum_j w[j][c] * u_(t - taps + 1 + j),   zeros before position 0
+// (the weights arrive tap-major, [taps, C], so that neighbouring channels are neighbouring loads).
 // A token whose tap reaches before the step's first row of its sequence reads the carried inputs; a
 // sequence that starts at position 0 ignores what its slot holds.
 //
@@ -30,15 +31,15 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ 
   const int li = (int)t - cu[s];  // index inside the step's portion
   const int p0 = start[s];        // position of the portion's first token
   const float* st = state + (int64_t)sslot[s] * (taps - 1) * C;
-  const float* wc = w + (int64_t)c * taps;
+  const float* wc = w + c;  // tap j of this channel: wc[j * C]
   const float cur = ldf(u + t * u_stride + c);
-  float acc = wc[taps - 1] * cur;
+  float acc = wc[(int64_t)(taps - 1) * C] * cur;
   for (int k = 1; k < taps; ++k) {
     const int i = li - k;
     float v = 0.f;
     if (i >= 0) v = ldf(u + (t - k) * u_stride + c);
     else if (p0 + i >= 0) v = st[(int64_t)(taps - 1 + i) * C + c];
-    acc += wc[taps - 1 - k] * v;
+    acc += wc[(int64_t)(taps - 1 - k) * C] * v;
   }
   if (add_input) acc += cur;
   stf(y + t * y_stride + c, acc);
@@ -58,10 +59,12 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(const T* __restric
   const int li = (int)t - cu[s];
   const int p0 = start[s];
   const float* st = state + (int64_t)sslot[s] * (taps - 1) * C;
-  float cur[N], acc[N], v[N];
+  float cur[N], acc[N], v[N], wk[N];
   Vec16<T>::load(u + t * u_stride + c, cur);
 #pragma unroll
-  for (int i = 0; i < N; ++i) acc[i] = w[(int64_t)(c + i) * taps + taps - 1] * cur[i];
+  for (int i = 0; i < N; i += 4) Vec16<float>::load(w + (int64_t)(taps - 1) * C + c + i, wk + i);
+#pragma unroll
+  for (int i = 0; i < N; ++i) acc[i] = wk[i] * cur[i];
   for (int k = 1; k < taps; ++k) {
     const int i0 = li - k;
     if (i0 >= 0) {
@@ -73,7 +76,9 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(const T* __restric
       continue;
     }
 #pragma unroll
-    for (int i = 0; i < N; ++i) acc[i] += w[(int64_t)(c + i) * taps + taps - 1 - k] * v[i];
+    for (int i = 0; i < N; i += 4) Vec16<float>::load(w + (int64_t)(taps - 1 - k) * C + c + i, wk + i);
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] += wk[i] * v[i];
   }
   if (add_input) {
 #pragma unroll
@@ -99,12 +104,12 @@ __global__ __launch_bounds__(256) void causal_conv_short_kernel(const T* __restr
   float* st = state + (int64_t)sslot[s] * (taps - 1) * C;
   float h[CONV_MAX_TAPS];  // h[j]: the input taps - 1 - j positions before the current token (h[taps-1] = current)
   for (int j = 0; j < taps - 1; ++j) h[j] = (p0 - (taps - 1) + j >= 0) ? st[(int64_t)j * C + c] : 0.f;
-  const float* wc = w + (int64_t)c * taps;
+  const float* wc = w + c;
   for (int i = 0; i < n; ++i) {
     const float cur = ldf(u + (int64_t)(a + i) * u_stride + c);
     h[taps - 1] = cur;
     float acc = add_input ? cur : 0.f;
-    for (int j = 0; j < taps; ++j) acc += wc[j] * h[j];
+    for (int j = 0; j < taps; ++j) acc += wc[(int64_t)j * C] * h[j];
     stf(y + (int64_t)(a + i) * C + c, acc);
     for (int j = 0; j < taps - 1; ++j) h[j] = h[j + 1];
   }
@@ -138,8 +143,8 @@ at::Tensor causal_conv(const at::Tensor& u, const at::Tensor& w, at::Tensor stat
                        const at::Tensor& start, const at::Tensor& sslot, bool add_input, int64_t max_len) {
   check_rows(u, "u");
   const int64_t T = u.size(0), C = u.size(1);
-  HYB_CHECK(w.is_cuda() && w.dim() == 2 && w.is_contiguous() && w.scalar_type() == at::kFloat && w.size(0) == C, "w: contiguous fp32 [C, taps]");
-  const int64_t taps = w.size(1);
+  HYB_CHECK(w.is_cuda() && w.dim() == 2 && w.is_contiguous() && w.scalar_type() == at::kFloat && w.size(1) == C, "w: contiguous fp32 [taps, C]");
+  const int64_t taps = w.size(0);
   HYB_CHECK(taps >= 1 && taps <= CONV_MAX_TAPS, "taps in [1, 16]");
   HYB_CHECK(state.is_cuda() && state.is_contiguous() && state.scalar_type() == at::kFloat && state.dim() == 3 && state.size(1) == taps - 1 && state.size(2) == C,
             "state: contiguous fp32 [slots, taps - 1, C]");
@@ -161,7 +166,7 @@ at::Tensor causal_conv(const at::Tensor& u, const at::Tensor& w, at::Tensor stat
       return;
     }
     constexpr int N = Vec16<Tt>::N;
-    if (C % 8 == 0 && aligned16<Tt>(u) && reinterpret_cast<uintptr_t>(state.data_ptr()) % 16 == 0)
+    if (C % 8 == 0 && aligned16<Tt>(u) && reinterpret_cast<uintptr_t>(state.data_ptr()) % 16 == 0 && reinterpret_cast<uintptr_t>(w.data_ptr()) % 16 == 0)
       causal_conv_vec_kernel<Tt><<<dim3((unsigned)T, (unsigned)((C / N + 255) / 256)), 256, 0, cur_stream()>>>(
           (const Tt*)u.data_ptr(), u.stride(0), w.data_ptr<float>(), state.data_ptr<float>(), seq_of.data_ptr<int>(), cu.data_ptr<int>(),
           start.data_ptr<int>(), sslot.data_ptr<int>(), (Tt*)y.data_ptr(), (int)C, (int)taps, add_input ? 1 : 0);

@@ -129,8 +129,8 @@ def clamped_glu(gu, limit: float, alpha: float):
 
 
 def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input: bool, max_len: int = 0):
-    """Short causal convolution over time per channel of the packed rows ``u [T, C]`` (``w`` fp32
-    ``[C, taps]``): ``y_t = (u_t if add_input) + sum_j w[:, j] u_(t - taps + 1 + j)``.  ``state`` (fp32
+    """Short causal convolution over time per channel of the packed rows ``u [T, C]`` (``w`` fp32, tap-major
+    ``[taps, C]``): ``y_t = (u_t if add_input) + sum_j w[j] u_(t - taps + 1 + j)``.  ``state`` (fp32
     ``[slots, taps - 1, C]``) carries each live sequence's last ``taps - 1`` inputs between steps (read
     at ``sslot[seq]`` unless the sequence starts at position 0, then updated in place).  ``max_len``: the
     longest portion of the step if the host knows it (steps of short portions take a one-launch form)."""

@@ -122,11 +122,11 @@ def clamped_glu(gu, limit, alpha):
 
 
 def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input):
-    """y_t = (u_t if add_input) + sum_j w[:, j] u_(t - taps + 1 + j) per sequence of the packed rows; the
+    """y_t = (u_t if add_input) + sum_j w[j] u_(t - taps + 1 + j) (w tap-major [taps, C]) per sequence of the packed rows; the
     last taps - 1 inputs of a sequence live in ``state[slot]`` ([taps - 1, C], oldest first) between steps
     and are ignored by a sequence that starts at position 0."""
     T, C = u.shape
-    taps = w.shape[1]
+    taps = w.shape[0]
     y = torch.zeros(T, C, dtype=torch.float32)
     cu_l = [int(v) for v in cu]
     for s in range(len(cu_l) - 1):
@@ -141,7 +141,7 @@ def causal_conv(u, w, state, seq_of, cu, start, sslot, add_input):
         n = b - a
         acc = torch.zeros(n, C)
         for j in range(taps):
-            acc += ext[j:j + n] * w[:, j].float()
+            acc += ext[j:j + n] * w[j].float()
         y[a:b] = acc + (u[a:b].float() if add_input else 0.0)
         if taps > 1:
             state[slot] = ext[-(taps - 1):]

@@ -227,7 +227,8 @@ class InferenceEngine:
                           p_bt=i32(pp["bt"]) if Tp else None, d_ctx=i32(dp["ctx"]) if Td else None,
                           d_bt=i32(dp["bt"]) if Td else None, cu=i32(cu), start=i32(start), state=i32(state),
                           max_q=max((b - a for a, b in zip(p_cu[:-1], p_cu[1:])), default=0), cu_host=cu,
-                          seq_of=i32(seq_of), d_max_ctx=int(max(dp["ctx"])) if Td else 0)
+                          seq_of=i32(seq_of), d_max_ctx=int(max(dp["ctx"])) if Td else 0,
+                          fresh=Td == 0 and all(int(v) == 0 for v in start))
         if rows is None:
             rows = (list(pp["last"]) if Tp else []) + list(range(Tp, Tp + Td))
         if count:

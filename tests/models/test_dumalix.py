@@ -93,6 +93,19 @@ def test_latent_attention_one_head_no_scaling(tmp_path, dev):
     check(tmp_path, dev, cfg, r, whole(r))
 
 
+@pytest.mark.parametrize("sizes", [dict(heads=3, dim=6, rot_dim=4, vdim=5, kv_rank=40), dict(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=64),
+                                   dict(heads=1, dim=2, rot_dim=2, vdim=2, kv_rank=9)])
+def test_latent_attention_whole_prompts_on_expanded_keys(tmp_path, dev, sizes, monkeypatch):
+    # whole prompts attend per-head keys and values expanded from the latents (a wide latent makes that the
+    # cheaper product); the second request runs in portions, which attend the cached rows, in the same steps
+    from llmctl.models.mixers import LatentAttention
+
+    monkeypatch.setattr(LatentAttention, "EXPAND_MIN_TOKENS", 1)
+    cfg = U.config([(U.lat(**sizes), U.ff()), (U.lat(**sizes), None)], taps=2)
+    r = {"a": tokens(70, 50, 40), "b": tokens(33, 50, 41), "c": tokens(21, 50, 42)}
+    check(tmp_path, dev, cfg, r, [[("a", 70), ("b", 20)], [("b", 13)], [("c", 21)]], blocks=40)
+
+
 def test_feed_forward_alone(tmp_path, dev):
     # the mixer sees one position only, so the clamped feed-forward carries the test; the limit is low
     # enough that both clamps bite
@@ -335,7 +348,7 @@ def _conv_case(device, dtype, C, taps, portions, residual, hint=True):
         seq_of = torch.repeat_interleave(torch.arange(len(seqs), dtype=torch.int32), torch.tensor([n for _, n in seqs]))
         start = torch.tensor([at[s] for s, _ in seqs], dtype=torch.int32)
         slot = torch.tensor([2 - s for s, _ in seqs], dtype=torch.int32)
-        y = hybrid.causal_conv(rows.to(d), w.to(d), state, seq_of.to(d), cu.to(d), start.to(d), slot.to(d), residual,
+        y = hybrid.causal_conv(rows.to(d), w.t().contiguous().to(d), state, seq_of.to(d), cu.to(d), start.to(d), slot.to(d), residual,
                                max_len=max(pa, pb) if hint else 0).cpu()
         o = 0
         for s, n in seqs:
