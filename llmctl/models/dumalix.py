@@ -308,9 +308,16 @@ class DumalixLM(nn.Module):
 def load_dumalix(ck: Path, cfg: DumalixConfig, device=None, dtype=torch.bfloat16) -> DumalixLM:
     from safetensors import safe_open
 
-    model = DumalixLM(cfg, device=device, dtype=dtype)
     with safe_open(str(ck / "model.safetensors"), framework="pt", device="cpu") as f:
         W = {k: f.get_tensor(k) for k in f.keys()}
+    # the convolutions' tap counts are the tensors' second size; they win over (or stand in for) the config's
+    if "l0.canon1" in W:
+        cfg.canon_taps = int(W["l0.canon1"].shape[1])
+    for i, spec in enumerate(cfg.layer_specs):
+        if spec["type"] == "attention":
+            w = W.get(f"l{i}.mix.q.conv")
+            spec["mixer"]["conv"] = int(w.shape[1]) if w is not None else 0
+    model = DumalixLM(cfg, device=device, dtype=dtype)
     model.load_named(W)
     return model
 
@@ -323,7 +330,7 @@ def dumalix_template(width: int = 256, layers: int = 4, heads: int = 4, kv_heads
     d = head_dim or width // heads
     rot = max(d // 2, 2) // 2 * 2
     yarn = {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}
-    lat = {"heads": heads, "dim": d, "rot_dim": rot, "vdim": d, "kv_rank": max(width // 4, 8),
+    lat = {"heads": heads, "dim": d, "rot_dim": rot, "vdim": d, "kv_rank": min(max(width // 4, 8), 512),
            "rot": {"base": 10000.0, "dims": rot, "scaling": dict(yarn)}, "scale": (d + rot) ** -0.5}
     att = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "conv": taps, "mask": {"size": chunk},
            "rot": {"base": 500000.0, "dims": d // 2 * 2, "scaling": dict(yarn)}, "scale": d ** -0.5}

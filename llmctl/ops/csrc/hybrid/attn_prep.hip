@@ -7,7 +7,7 @@
 //   v      optionally turned the same way over all of dv by position * vfreq[m] (the attention
 //          kernel turns the head's weighted sum back by the query's position);
 //   k, v   written to the token's cache row of kv head g: [v (dv) | k (dk)]; q returned [T, H, dk].
-// One workgroup per token, one wave per head slot in turn; all arithmetic fp32.  The token's cos / sin
+// One workgroup per token (up to 16 waves), one wave per head slot in turn; all arithmetic fp32.  The token's cos / sin
 // (they depend on the position and the pair only) are computed once into LDS and shared by its heads.
 #include "hybrid_common.h"
 
@@ -25,7 +25,7 @@ __device__ __forceinline__ void pair_idx(int p, int dims, bool inter, int& i0, i
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict__ z, int64_t z_stride, const float* __restrict__ qn,
+__global__ __launch_bounds__(1024) void attn_qkv_prep_kernel(const T* __restrict__ z, int64_t z_stride, const float* __restrict__ qn,
                                                             const float* __restrict__ kn, const int* __restrict__ pos,
                                                             const float* __restrict__ freq, const float* __restrict__ vfreq,
                                                             T* __restrict__ q_out, T* __restrict__ cache,
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict_
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float p = (float)pos[t];
   const int nrot = rot_dims / 2, nv = vfreq != nullptr ? dv / 2 : 0;
-  for (int i = threadIdx.x; i < nrot + nv; i += 256) {
+  for (int i = threadIdx.x; i < nrot + nv; i += blockDim.x) {
     float s, c;
     if (i < nrot) {
       sincosf(p * freq[i], &s, &c);
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const T* __restrict_
   const int64_t slot = slots[t];
   const int rs = dv + dk;
   const T* zr = z + t * z_stride;
-  for (int hs = wave; hs < H + 2 * G; hs += 4) {
+  for (int hs = wave; hs < H + 2 * G; hs += (int)(blockDim.x >> 6)) {
     if (hs < H + G) {  // a query or key head: norm, rotary
       const bool is_q = hs < H;
       const T* x = zr + (int64_t)hs * dk;  // k heads follow the q heads at the same pitch
@@ -116,7 +116,8 @@ at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, 
   if (T == 0) return q;
   dispatch_act(z, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), 256, (size_t)(rot_dims + dv) * sizeof(float), cur_stream()>>>(
+    const unsigned nthreads = (unsigned)std::min<int64_t>(16, std::max<int64_t>(4, H + 2 * G)) * 64;
+    attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), nthreads, (size_t)(rot_dims + dv) * sizeof(float), cur_stream()>>>(
         (const Tt*)z.data_ptr(), z.stride(0), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), pos.data_ptr<int>(), freq.data_ptr<float>(),
         vfreq.has_value() ? vfreq->data_ptr<float>() : nullptr, (Tt*)q.data_ptr(), (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)H,
         (int)G, (int)dk, (int)dv, (int)rot_dims, interleaved ? 1 : 0, (float)amp, (float)eps);

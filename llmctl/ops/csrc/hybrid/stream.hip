@@ -47,10 +47,28 @@ __global__ __launch_bounds__(NT) void add_rmsnorm2_kernel(float* __restrict__ x,
                                                           const float* __restrict__ w2, T* __restrict__ h1, T* __restrict__ h2, int W,
                                                           float eps, float plus) {
   __shared__ float red[NW];
+  constexpr int KEEP = 16;  // a thread's first KEEP values stay in registers (rows up to KEEP * NT wide are read once)
   const int64_t r = blockIdx.x;
   float* xr = x + r * W;
+  float keep[KEEP];
   float q = 0.f;
-  for (int c = threadIdx.x; c < W; c += NT) {
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int c = threadIdx.x + i * NT;
+    float v = 0.f;
+    if (c < W) {
+      v = xr[c];
+      if (a != nullptr) {
+        float d = ldf(a + r * a_stride + c);
+        if (b != nullptr) d += ldf(b + r * b_stride + c);
+        v += d;
+        xr[c] = v;
+      }
+    }
+    keep[i] = v;
+    q += v * v;
+  }
+  for (int c = threadIdx.x + KEEP * NT; c < W; c += NT) {
     float v = xr[c];
     if (a != nullptr) {
       float d = ldf(a + r * a_stride + c);
@@ -62,7 +80,16 @@ __global__ __launch_bounds__(NT) void add_rmsnorm2_kernel(float* __restrict__ x,
   }
   if (h1 == nullptr) return;
   const float rstd = 1.0f / sqrtf(block_sum<NW>(q, red) / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += NT) {
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < W) {
+      const float v = keep[i] * rstd;
+      stf(h1 + r * W + c, v * (plus + w1[c]));
+      if (h2 != nullptr) stf(h2 + r * W + c, v * (plus + w2[c]));
+    }
+  }
+  for (int c = threadIdx.x + KEEP * NT; c < W; c += NT) {
     const float v = xr[c] * rstd;
     stf(h1 + r * W + c, v * (plus + w1[c]));
     if (h2 != nullptr) stf(h2 + r * W + c, v * (plus + w2[c]));
