@@ -116,7 +116,8 @@ at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, 
   if (T == 0) return q;
   dispatch_act(z, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
-    const unsigned nthreads = (unsigned)std::min<int64_t>(16, std::max<int64_t>(4, H + 2 * G)) * 64;
+    // few tokens (decode steps): one wave per head slot, up to 16; many tokens: 4 waves per token fill the chip
+    const unsigned nthreads = T >= 256 ? 256u : (unsigned)std::min<int64_t>(16, std::max<int64_t>(4, H + 2 * G)) * 64;
     attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), nthreads, (size_t)(rot_dims + dv) * sizeof(float), cur_stream()>>>(
         (const Tt*)z.data_ptr(), z.stride(0), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), pos.data_ptr<int>(), freq.data_ptr<float>(),
         vfreq.has_value() ? vfreq->data_ptr<float>() : nullptr, (Tt*)q.data_ptr(), (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)H,
