@@ -28,10 +28,10 @@ SIZES = {
 # Dumalix: width, layers (every third is chunked grouped-query attention, the others latent attention),
 # loop (start, stop, times), heads of 128, kv heads, feed-forward, chunk, prompt, decode batch
 DUMALIX_SIZES = {
-    "tiny": dict(width=128, layers=3, loop=(1, 3, 2), heads=4, kv_heads=2, head_dim=32, ff=192, chunk=32, prompt=64, batch=2),
-    "small": dict(width=1024, layers=6, loop=(1, 3, 2), heads=8, kv_heads=2, head_dim=128, ff=3072, chunk=1024, prompt=2048, batch=16),
-    "medium": dict(width=2048, layers=6, loop=(1, 3, 2), heads=16, kv_heads=4, head_dim=128, ff=6144, chunk=1024, prompt=2048, batch=16),
-    "large": dict(width=4096, layers=6, loop=(1, 3, 2), heads=32, kv_heads=8, head_dim=128, ff=12288, chunk=2048, prompt=4096, batch=16),
+    "tiny": dict(width=128, layers=3, loop=(1, 2, 2), heads=4, kv_heads=2, head_dim=32, ff=192, chunk=32, prompt=64, batch=2),
+    "small": dict(width=1024, layers=6, loop=(2, 5, 2), heads=8, kv_heads=2, head_dim=128, ff=3072, chunk=1024, prompt=2048, batch=16),
+    "medium": dict(width=2048, layers=6, loop=(2, 5, 2), heads=16, kv_heads=4, head_dim=128, ff=6144, chunk=1024, prompt=2048, batch=16),
+    "large": dict(width=4096, layers=6, loop=(2, 5, 2), heads=32, kv_heads=8, head_dim=128, ff=12288, chunk=2048, prompt=4096, batch=16),
 }
 
 

@@ -150,7 +150,7 @@ def test_stream_after_every_run(tmp_path, dev):
 def test_yarn_frequencies():
     from llmctl.models.mixers import rotary_frequencies
 
-    for base, dims, sc in [(10000.0, 16, {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}),
+    for base, dims, sc in [(20000.0, 24, {"factor": 6.0, "original": 4096, "fast": 16.0, "slow": 2.0}),
                            (50.0, 8, U.YARN), (500000.0, 64, {"factor": 2.0, "original": 100, "fast": 8.0, "slow": 2.0}),
                            (100.0, 6, None), (3.0, 4, {"factor": 5.0, "original": 4, "fast": 1.0, "slow": 1.0})]:
         f, amp = rotary_frequencies(base, dims, sc)
@@ -288,7 +288,7 @@ def _edge_case(device, dtype, chunk, bs, L, j0, form, mfma=True, H=4, G=2, dk=8,
 
 @pytest.mark.parametrize("form", ["prefill", "decode"])
 @pytest.mark.parametrize("chunk,bs,L,j0", [(5, 4, 20, 14), (5, 4, 20, 15), (8, 8, 40, 31), (8, 8, 40, 32), (70, 16, 200, 139),
-                                           (70, 16, 200, 140), (64, 16, 200, 191), (64, 16, 200, 192), (200, 16, 420, 399), (200, 16, 420, 400),
+                                           (70, 16, 200, 140), (64, 16, 200, 191), (64, 16, 200, 192), (136, 16, 420, 407), (136, 16, 420, 408),
                                            (1000, 16, 700, 3), (300, 16, 700, 600)])
 def test_chunk_edges_and_far_keys(dev, form, chunk, bs, L, j0):
     device, dtype, _ = dev
@@ -299,7 +299,7 @@ def test_chunk_edges_and_far_keys(dev, form, chunk, bs, L, j0):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,G,dk,dv,chunk", [(8, 2, 48, 48, 200), (4, 4, 64, 32, 33), (6, 1, 128, 128, 1000), (3, 3, 24, 40, 64),
+@pytest.mark.parametrize("H,G,dk,dv,chunk", [(8, 4, 56, 40, 210), (4, 4, 64, 32, 33), (6, 1, 128, 128, 1000), (3, 3, 24, 40, 64),
                                             (2, 1, 7, 10, 50), (16, 2, 16, 264, 90)])
 def test_grouped_attention_kernels_gpu(H, G, dk, dv, chunk):
     # random rows, every kernel form against full scores with an explicit mask
