@@ -117,7 +117,7 @@ class DumalixConfig:
 def _attention(width, m, eps, **kw):
     rot = m["rot"]
     return GroupedAttention(width, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
-                            vdim=int(m["vdim"]), rot_base=float(rot["base"]), rot_dims=int(rot["dims"]),
+                            vdim=int(m["vdim"]), rot_base=float(rot["base"]), rot_dims=int(rot.get("dims", m["dim"])),
                             scale=float(m["scale"]), eps=eps, conv_taps=int(m.get("conv") or 0),
                             rot_scaling=rot.get("scaling"), interleaved=True, rotate_values=True, temperature=True,
                             chunk=(m.get("mask") or {}).get("size"), sink=True, **kw)

@@ -97,6 +97,110 @@ __global__ __launch_bounds__(1024) void attn_qkv_prep_kernel(const T* __restrict
   }
 }
 
+// Two neighbours at once: one 4-byte (bf16) or 8-byte (fp32) access
+template <typename T>
+struct Pair;
+template <>
+struct Pair<bf16_t> {
+  __device__ __forceinline__ static void ld(const bf16_t* p, float& a, float& b) {
+    const unsigned w = *reinterpret_cast<const unsigned*>(p);
+    a = __uint_as_float(w << 16);
+    b = __uint_as_float(w & 0xffff0000u);
+  }
+  __device__ __forceinline__ static void st(bf16_t* p, float a, float b) {
+    *reinterpret_cast<unsigned*>(p) =
+        (unsigned)__bfloat16_as_ushort(__float2bfloat16(a)) | ((unsigned)__bfloat16_as_ushort(__float2bfloat16(b)) << 16);
+  }
+};
+template <>
+struct Pair<float> {
+  __device__ __forceinline__ static void ld(const float* p, float& a, float& b) {
+    const float2 w = *reinterpret_cast<const float2*>(p);
+    a = w.x;
+    b = w.y;
+  }
+  __device__ __forceinline__ static void st(float* p, float a, float b) { *reinterpret_cast<float2*>(p) = make_float2(a, b); }
+};
+
+// The form for many tokens, neighbour pairs and heads of at most 128: lane p owns pair (2p, 2p+1) of a head, a wave first
+// requests the pairs of up to eight head slots (so that eight loads per lane are in flight), then norms, turns
+// and stores them.  Same arithmetic as the kernel above.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_qkv_prep_pairs_kernel(const T* __restrict__ z, int64_t z_stride, const float* __restrict__ qn,
+                                                                  const float* __restrict__ kn, const int* __restrict__ pos,
+                                                                  const float* __restrict__ freq, const float* __restrict__ vfreq,
+                                                                  T* __restrict__ q_out, T* __restrict__ cache,
+                                                                  const int64_t* __restrict__ slots, int H, int G, int dk, int dv,
+                                                                  int rot_dims, float amp, float eps) {
+  extern __shared__ float cs_tab[];
+  constexpr int MAXS = 8;
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float p = (float)pos[t];
+  const int nrot = rot_dims / 2, nv = vfreq != nullptr ? dv / 2 : 0;
+  for (int i = threadIdx.x; i < nrot + nv; i += 256) {
+    float s, c;
+    if (i < nrot) {
+      sincosf(p * freq[i], &s, &c);
+      s *= amp;
+      c *= amp;
+    } else {
+      sincosf(p * vfreq[i - nrot], &s, &c);
+    }
+    cs_tab[2 * i] = c;
+    cs_tab[2 * i + 1] = s;
+  }
+  __syncthreads();
+  const int64_t slot = slots[t];
+  const int rs = dv + dk, nslots = H + 2 * G;
+  const T* zr = z + t * z_stride;
+  for (int base = 0; base < nslots; base += 4 * MAXS) {
+    float xa[MAXS], xb[MAXS];
+#pragma unroll
+    for (int k = 0; k < MAXS; ++k) {
+      const int hs = base + wave + 4 * k;
+      xa[k] = 0.f;
+      xb[k] = 0.f;
+      if (hs < nslots) {
+        const bool qk = hs < H + G;
+        const T* x = qk ? zr + (int64_t)hs * dk : zr + (int64_t)(H + G) * dk + (int64_t)(hs - H - G) * dv;
+        if (2 * lane < (qk ? dk : dv)) Pair<T>::ld(x + 2 * lane, xa[k], xb[k]);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < MAXS; ++k) {
+      const int hs = base + wave + 4 * k;  // the same for every lane of the wave
+      if (hs >= nslots) continue;
+      float a = xa[k], b = xb[k];
+      if (hs < H + G) {
+        const bool is_q = hs < H;
+        const float rstd = 1.0f / sqrtf(wave_sum(a * a + b * b) / (float)dk + eps);
+        if (2 * lane >= dk || (!is_q && slot < 0)) continue;
+        const float* nw = is_q ? qn : kn;
+        a *= rstd * nw[2 * lane];
+        b *= rstd * nw[2 * lane + 1];
+        if (lane < nrot) {
+          const float c = cs_tab[2 * lane], sn = cs_tab[2 * lane + 1];
+          const float ra = a * c - b * sn, rb = b * c + a * sn;
+          a = ra;
+          b = rb;
+        }
+        T* out = is_q ? q_out + (t * H + hs) * dk : cache + (slot * G + (hs - H)) * rs + dv;
+        Pair<T>::st(out + 2 * lane, a, b);
+      } else {
+        if (2 * lane >= dv || slot < 0) continue;
+        if (vfreq != nullptr) {
+          const float c = cs_tab[2 * (nrot + lane)], sn = cs_tab[2 * (nrot + lane) + 1];
+          const float ra = a * c - b * sn, rb = b * c + a * sn;
+          a = ra;
+          b = rb;
+        }
+        Pair<T>::st(cache + (slot * G + (hs - H - G)) * rs + 2 * lane, a, b);
+      }
+    }
+  }
+}
+
 at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, int64_t dv, const at::Tensor& q_norm,
                          const at::Tensor& k_norm, double eps, const at::Tensor& pos, const at::Tensor& freq, int64_t rot_dims,
                          bool interleaved, double amp, const c10::optional<at::Tensor>& vfreq, at::Tensor cache, const at::Tensor& slots) {
@@ -116,6 +220,14 @@ at::Tensor attn_qkv_prep(const at::Tensor& z, int64_t H, int64_t G, int64_t dk, 
   if (T == 0) return q;
   dispatch_act(z, [&](auto* tag) {
     using Tt = std::remove_pointer_t<decltype(tag)>;
+    if (T >= 256 && interleaved && dk % 2 == 0 && dv % 2 == 0 && dk <= 128 && dv <= 128 && z.stride(0) % 2 == 0 &&
+        reinterpret_cast<uintptr_t>(z.data_ptr()) % 8 == 0) {
+      attn_qkv_prep_pairs_kernel<Tt><<<dim3((unsigned)T), 256, (size_t)(rot_dims + dv) * sizeof(float), cur_stream()>>>(
+          (const Tt*)z.data_ptr(), z.stride(0), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), pos.data_ptr<int>(), freq.data_ptr<float>(),
+          vfreq.has_value() ? vfreq->data_ptr<float>() : nullptr, (Tt*)q.data_ptr(), (Tt*)cache.data_ptr(), slots.data_ptr<int64_t>(), (int)H,
+          (int)G, (int)dk, (int)dv, (int)rot_dims, (float)amp, (float)eps);
+      return;
+    }
     // few tokens (decode steps): one wave per head slot, up to 16; many tokens: 4 waves per token fill the chip
     const unsigned nthreads = T >= 256 ? 256u : (unsigned)std::min<int64_t>(16, std::max<int64_t>(4, H + 2 * G)) * 64;
     attn_qkv_prep_kernel<Tt><<<dim3((unsigned)T), nthreads, (size_t)(rot_dims + dv) * sizeof(float), cur_stream()>>>(

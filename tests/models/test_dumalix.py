@@ -310,6 +310,45 @@ def test_grouped_attention_kernels_gpu(H, G, dk, dv, chunk):
                 assert float((got - want).abs().max()) < tol, (dtype, form, mfma)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("T", [20, 300])
+@pytest.mark.parametrize("H,G,dk,dv,rot_dims", [(6, 2, 32, 48, 32), (4, 4, 128, 64, 96), (3, 1, 10, 6, 4), (40, 8, 16, 16, 16), (2, 1, 160, 136, 160)])
+def test_qkv_preparation_kernels_gpu(T, H, G, dk, dv, rot_dims):
+    # both kernel forms (few rows: a wave per head; many rows: a lane per pair) against the plain functions
+    from llmctl.models.mixers import rotary_frequencies
+    from llmctl.ops import hybrid
+
+    g = torch.Generator().manual_seed(11)
+    d = torch.device("cuda")
+    z = torch.randn(T, (H + G) * dk + G * dv, generator=g)
+    qn, kn = 1.0 + 0.2 * torch.randn(dk, generator=g), 1.0 + 0.2 * torch.randn(dk, generator=g)
+    pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(T + 7, generator=g)[:T]
+    rot = {"base": 3000.0, "dims": rot_dims, "scaling": {"factor": 5.0, "original": 64, "fast": 8.0, "slow": 1.0}}
+    freq, amp = rotary_frequencies(rot["base"], rot_dims, rot["scaling"])
+    vfreq, _ = rotary_frequencies(rot["base"], dv, None)
+    zd = z.double()
+    q = plain.rotary(plain.norm_plain(zd[:, :H * dk].view(T, H, dk), qn, 1e-5), pos, rot)
+    k = plain.rotary(plain.norm_plain(zd[:, H * dk:(H + G) * dk].view(T, G, dk), kn, 1e-5), pos, rot)
+    v = plain.turn_pairs(zd[:, (H + G) * dk:].view(T, G, dv), pos.double()[:, None, None] * vfreq.double())
+    for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 3e-2)):
+        zt = z.to(dtype)
+        if dtype == torch.bfloat16:
+            continue_ref = zt.double()
+            q2 = plain.rotary(plain.norm_plain(continue_ref[:, :H * dk].view(T, H, dk), qn, 1e-5), pos, rot)
+            k2 = plain.rotary(plain.norm_plain(continue_ref[:, H * dk:(H + G) * dk].view(T, G, dk), kn, 1e-5), pos, rot)
+            v2 = plain.turn_pairs(continue_ref[:, (H + G) * dk:].view(T, G, dv), pos.double()[:, None, None] * vfreq.double())
+        else:
+            q2, k2, v2 = q, k, v
+        cache = torch.zeros(T + 7, 1, G * (dv + dk), dtype=dtype, device=d)
+        got_q = hybrid.attn_qkv_prep(zt.to(d), H, G, dk, dv, qn.to(d), kn.to(d), 1e-5, pos.to(d), freq.to(d), rot_dims, True, amp,
+                                     vfreq.to(d), cache, slots.to(d))
+        rows = cache.view(T + 7, G, dv + dk)[slots.to(d)].double().cpu()
+        assert float((got_q.double().cpu() - q2).abs().max()) < tol * 4
+        assert float((rows[:, :, dv:] - k2).abs().max()) < tol * 4
+        assert float((rows[:, :, :dv] - v2).abs().max()) < tol * 4
+
+
 def test_output_turn_back():
     # ofreq turns the head outputs' neighbour pairs by minus the query's position
     from llmctl.ops import hybrid
