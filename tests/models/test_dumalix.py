@@ -324,22 +324,23 @@ def test_qkv_preparation_kernels_gpu(T, H, G, dk, dv, rot_dims):
     qn, kn = 1.0 + 0.2 * torch.randn(dk, generator=g), 1.0 + 0.2 * torch.randn(dk, generator=g)
     pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
     slots = torch.randperm(T + 7, generator=g)[:T]
-    rot = {"base": 3000.0, "dims": rot_dims, "scaling": {"factor": 5.0, "original": 64, "fast": 8.0, "slow": 1.0}}
-    freq, amp = rotary_frequencies(rot["base"], rot_dims, rot["scaling"])
-    vfreq, _ = rotary_frequencies(rot["base"], dv, None)
-    zd = z.double()
-    q = plain.rotary(plain.norm_plain(zd[:, :H * dk].view(T, H, dk), qn, 1e-5), pos, rot)
-    k = plain.rotary(plain.norm_plain(zd[:, H * dk:(H + G) * dk].view(T, G, dk), kn, 1e-5), pos, rot)
-    v = plain.turn_pairs(zd[:, (H + G) * dk:].view(T, G, dv), pos.double()[:, None, None] * vfreq.double())
+    freq, amp = rotary_frequencies(3000.0, rot_dims, {"factor": 5.0, "original": 64, "fast": 8.0, "slow": 1.0})
+    vfreq, _ = rotary_frequencies(3000.0, dv, None)
+    # angles as the kernels form them: the fp32 product of position and frequency (at positions in the
+    # thousands its rounding, ~1e-4 rad, is far above the bound that the comparison can then keep)
+    ang = (pos.float()[:, None, None] * freq[None, None, :]).double()
+    vang = (pos.float()[:, None, None] * vfreq[None, None, :]).double()
+
+    def expect(zz):
+        zz = zz.double()
+        turn = lambda x: torch.cat([plain.turn_pairs(x[..., :rot_dims], ang, amp), x[..., rot_dims:]], -1)
+        return (turn(plain.norm_plain(zz[:, :H * dk].view(T, H, dk), qn, 1e-5)),
+                turn(plain.norm_plain(zz[:, H * dk:(H + G) * dk].view(T, G, dk), kn, 1e-5)),
+                plain.turn_pairs(zz[:, (H + G) * dk:].view(T, G, dv), vang))
+
     for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 3e-2)):
         zt = z.to(dtype)
-        if dtype == torch.bfloat16:
-            continue_ref = zt.double()
-            q2 = plain.rotary(plain.norm_plain(continue_ref[:, :H * dk].view(T, H, dk), qn, 1e-5), pos, rot)
-            k2 = plain.rotary(plain.norm_plain(continue_ref[:, H * dk:(H + G) * dk].view(T, G, dk), kn, 1e-5), pos, rot)
-            v2 = plain.turn_pairs(continue_ref[:, (H + G) * dk:].view(T, G, dv), pos.double()[:, None, None] * vfreq.double())
-        else:
-            q2, k2, v2 = q, k, v
+        q2, k2, v2 = expect(zt)
         cache = torch.zeros(T + 7, 1, G * (dv + dk), dtype=dtype, device=d)
         got_q = hybrid.attn_qkv_prep(zt.to(d), H, G, dk, dv, qn.to(d), kn.to(d), 1e-5, pos.to(d), freq.to(d), rot_dims, True, amp,
                                      vfreq.to(d), cache, slots.to(d))
