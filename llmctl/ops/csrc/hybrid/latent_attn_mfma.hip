@@ -70,7 +70,8 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int qlen = a.cu ? a.cu[n + 1] - q_begin : 1;
   const int HB = a.HB, TB = 128 / HB;
   const int split = a.nsplit > 1 ? blockIdx.x : 0;
-  const int tok0 = a.nsplit > 1 ? 0 : blockIdx.x * TB;
+  // prompt portions: the last query blocks of a sequence see the most keys; they are dispatched first
+  const int tok0 = a.nsplit > 1 ? 0 : (int)(gridDim.x - 1 - blockIdx.x) * TB;
   if (tok0 >= qlen) return;
   const int ctx = a.ctx[n];
   const int pos0 = ctx - qlen;
