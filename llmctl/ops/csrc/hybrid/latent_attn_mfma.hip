@@ -123,6 +123,13 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
   const int w_last = pos0 + min(tok0 + (wave * 32 + 31) / HB, qlen - 1);
   const bool wave_live = tok0 + (wave * 32) / HB < qlen && hsub + (HB >= 32 ? (wave * 32) % HB : 0) < P;
   const int w_lo = first_key(w_first), my_lo = first_key(my_pos);
+  const int w_lo_last = first_key(w_last);  // first_key never decreases with the position
+  // lane-only parts of the LDS read addresses, so that the key loop adds constants to them
+  int tr_lo[4], tr_hi[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) tr_frag_offs<128>(c * 32, lane, tr_lo[c], tr_hi[c]);
+  // K fragment of k-step ks, rows kb * 32 + r: chunk (2 ks + hh) ^ (r & 15) = (2 ks) ^ (hh ^ (r & 15))
+  const int k_row = r * LROWB, k_x = (hh ^ (r & 15)) << 4;
 
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const unsigned lds_base = lds_addr(smem);
@@ -199,21 +206,34 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        const bf16x8_t kf = lds_read_b128(Ks + (ks >> 3) * LIMG, row_off<128>(kb * 32 + r, (2 * ks + hh) & 15));
+        const bf16x8_t kf = lds_read_b128(Ks + (ks >> 3) * LIMG + kb * 32 * LROWB, k_row + (k_x ^ (((2 * ks) & 15) << 4)));
         s[kb] = mfma32(kf, qf[ks], s[kb]);
       }
     }
     float mx = -INFINITY;
+    if (kv0 + LKB - 1 <= w_first && kv0 >= w_lo_last && kv0 + LKB - 1 < ctx) {
+      // every key of the tile is visible to every row of this wave: no mask (rows past the portion's end
+      // carry finite scores of a repeated row and are never stored)
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float x = s[kb][i] * my_scale;
-        const int key = kv0 + kb * 32 + acc_row(i, hh);
-        if (!valid || key > my_pos || key < my_lo || key >= ctx) x = -INFINITY;
-        s[kb][i] = x;
-        mx = fmaxf(mx, x);
-      }
+        for (int i = 0; i < 16; ++i) {
+          s[kb][i] *= my_scale;
+          mx = fmaxf(mx, s[kb][i]);
+        }
+      if (!valid) mx = -INFINITY;  // such a row must not trigger the wave's rescale
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float x = s[kb][i] * my_scale;
+          const int key = kv0 + kb * 32 + acc_row(i, hh);
+          if (!valid || key > my_pos || key < my_lo || key >= ctx) x = -INFINITY;
+          s[kb][i] = x;
+          mx = fmaxf(mx, x);
+        }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const bool grow = __builtin_amdgcn_ballot_w64(mx > m_i + kRescaleTh) != 0;
     const float m_raw = grow ? fmaxf(m_i, mx) : m_i;
@@ -248,7 +268,7 @@ __global__ __launch_bounds__(256, 1) void latent_attn_mfma_kernel(LArgs a) {
       for (int st = 0; st < 2; ++st)
 #pragma unroll
         for (int d = 0; d < NDB; ++d) {
-          const bf16x8_t vf = tr_frag<128>(Vs + (d >> 2) * LIMG, kb * 32 + 16 * st, (d & 3) * 32, lane);
+          const bf16x8_t vf = tr_frag_at<128>(Vs + (d >> 2) * LIMG, kb * 32 + 16 * st, tr_lo[d & 3], tr_hi[d & 3]);
           o[d] = mfma32(vf, pb[kb][st], o[d]);
         }
   }
